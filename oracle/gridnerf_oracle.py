@@ -1,0 +1,283 @@
+"""CPU oracle for the GridNeRF render path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the product package may import this module: it exists so that tests,
+the smoke check and the benchmark's CPU-baseline leg can compare the HIP path
+with an independent restatement of the reference's PyTorch arithmetic.  Every
+function names the reference lines it follows (paths relative to the reference
+checkout).  The arithmetic itself lives in PyTorch (`F.grid_sample`,
+`torch.cumprod`, `F.softplus`, `F.linear`, `torch.linspace`, boolean-mask
+indexing), so the oracle issues the same ATen calls in the same order with the
+same operand dtypes: that is what makes the geometry / occupancy decisions
+reproducible bit for bit.
+
+How each function is pinned (tests/test_oracle_*.py):
+  sample_ray_aabb / sample_ray_within_hull   closed forms + brute force
+  sample_alpha                               scalar trilinear loop, volume invariants
+  normalize_coord                            AABB corners -> +-1
+  density_feature / app_feature              scalar bilinear loop, affine planes,
+                                             texel-centre queries, one-hot column order
+  feature2density                            library softplus / relu
+  raw2alpha                                  double-loop volume rendering, closed forms
+  positional_encoding                        math.sin / math.cos, index order
+  mlp_render                                 fp64 numpy matmul chain
+  render_chunk (composition order)           golden vectors written by
+                                             tests/golden/make_golden.py from the
+                                             reference's own forward
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+MAT_MODE = [[0, 1], [0, 2], [1, 2]]  # app/models/gridnerf_sequential.py:106
+VEC_MODE = [2, 1, 0]  # app/models/gridnerf_sequential.py:107
+
+
+# --------------------------------------------------------------------------------------
+# sampling
+# --------------------------------------------------------------------------------------
+def sample_ray_aabb(p, rays_o, rays_d, N_samples=-1):
+    """Equal-step samples from the slab entry point (sampling_opt=0, eval mode).
+
+    Follows app/models/gridnerf_sequential.py:260-281 with is_train=False.
+    Returns (pts [N,S,3], z [N,S], inside [N,S] bool).
+    """
+    S = N_samples if N_samples > 0 else p.nSamples
+    near, far = p.near_far
+    vec = torch.where(rays_d == 0, torch.full_like(rays_d, 1e-6), rays_d)
+    rate_a = (p.aabb[1] - rays_o) / vec
+    rate_b = (p.aabb[0] - rays_o) / vec
+    t_min = torch.minimum(rate_a, rate_b).amax(-1).clamp(min=near, max=far)
+    rng = torch.arange(S)[None].float()
+    step = p.stepSize * rng.to(rays_o.device)
+    z = t_min[..., None] + step
+    pts = rays_o[..., None, :] + rays_d[..., None, :] * z[..., None]
+    outside = ((p.aabb[0] > pts) | (pts > p.aabb[1])).any(dim=-1)
+    return pts, z, ~outside
+
+
+def sample_ray_within_hull(p, rays_o, rays_d, N_samples):
+    """Samples between `near` and the ray's hit with the AABB floor (sampling_opt=1).
+
+    Follows app/models/gridnerf_sequential.py:298-319 with is_train=False.
+    """
+    near, far = p.near_far
+    o_z = rays_o[:, -1:] - p.aabb[0, 2].item()
+    d_z = rays_d[:, -1:]
+    far = -(o_z / d_z)
+    far[rays_d[:, 2] >= 0] = p.near_far[-1]
+    t_vals = torch.linspace(0.0, 1.0, steps=N_samples, device=rays_o.device)
+    z = near * (1.0 - t_vals) + far * t_vals
+    pts = rays_o[..., None, :] + rays_d[..., None, :] * z[..., :, None]
+    outside = ((p.aabb[0] > pts) | (pts > p.aabb[1])).any(dim=-1)
+    return pts, z, ~outside
+
+
+# --------------------------------------------------------------------------------------
+# occupancy volume
+# --------------------------------------------------------------------------------------
+def sample_alpha(alpha_volume, alpha_aabb, pts):
+    """Trilinear lookup in the occupancy volume, app/models/alpha_mask.py:16-59.
+
+    `alpha_volume` is [D,H,W]; pts are world-space [M,3] (x->W, y->H, z->D).
+    """
+    size = alpha_aabb[1] - alpha_aabb[0]
+    inv = 1.0 / size * 2
+    c = (pts - alpha_aabb[0]) * inv - 1
+    vol = alpha_volume.view(1, 1, *alpha_volume.shape[-3:])
+    return F.grid_sample(vol, c.view(1, -1, 1, 1, 3), align_corners=True).view(-1)
+
+
+def normalize_coord(p, pts):
+    """app/models/gridnerf_sequential.py:203-204."""
+    return (pts - p.aabb[0]) * p.invaabbSize - 1
+
+
+# --------------------------------------------------------------------------------------
+# plane / line features
+# --------------------------------------------------------------------------------------
+def _coords(p, xyz):
+    """Grid-sample coordinate tensors, app/models/gridnerf_sequential.py:790-795."""
+    n = p.ndims
+    cp = torch.stack([xyz[..., MAT_MODE[i]] for i in range(n)]).view(n, -1, 1, 2)
+    cl = torch.stack([xyz[..., VEC_MODE[i]] for i in range(n)])
+    cl = torch.stack((torch.zeros_like(cl), cl), dim=-1).view(n, -1, 1, 2)
+    return cp, cl
+
+
+def _f32(t):
+    # fp16 plane storage is interpolated in fp32
+    # (app/models/gridnerf_tensor_parallel.py:74-81,180-181).
+    return t if t.dtype == torch.float32 else t.float()
+
+
+def density_feature(p, xyz):
+    """Sum over planes and channels of plane*line, gridnerf_sequential.py:790-827
+    (nonlinear_density=False, return_feat=False).  xyz is normalised [M,3]."""
+    cp, cl = _coords(p, xyz)
+    L = len(p.resMode)
+    out = torch.zeros((xyz.shape[0],), device=xyz.device)
+    for k in range(len(p.density_plane)):
+        d = k // L
+        pc = F.grid_sample(_f32(p.density_plane[k]), cp[[d]], align_corners=True).view(-1, xyz.shape[0])
+        lc = F.grid_sample(_f32(p.density_line[k]), cl[[d]], align_corners=True).view(-1, xyz.shape[0])
+        out = out + torch.sum(pc * lc, dim=0)
+    return out
+
+
+def app_products(p, xyz):
+    """[M, P*L*C_a] plane*line products; column = plane index major, channel minor
+    (gridnerf_sequential.py:846-864)."""
+    cp, cl = _coords(p, xyz)
+    L = len(p.resMode)
+    pcs, lcs = [], []
+    for k in range(len(p.app_plane)):
+        d = k // L
+        pcs.append(F.grid_sample(_f32(p.app_plane[k]), cp[[d]], align_corners=True).view(-1, xyz.shape[0]))
+        lcs.append(F.grid_sample(_f32(p.app_line[k]), cl[[d]], align_corners=True).view(-1, xyz.shape[0]))
+    return (torch.cat(pcs) * torch.cat(lcs)).T
+
+
+def app_feature(p, xyz):
+    """basis_mat(products), gridnerf_sequential.py:871 (Linear without bias, :678)."""
+    return F.linear(app_products(p, xyz), p.basis_mat)
+
+
+def feature2density(p, f):
+    """gridnerf_sequential.py:396-399."""
+    if p.fea2denseAct == "softplus":
+        return F.softplus(f + p.density_shift)
+    if p.fea2denseAct == "relu":
+        return F.relu(f)
+    raise ValueError(p.fea2denseAct)
+
+
+# --------------------------------------------------------------------------------------
+# compositing
+# --------------------------------------------------------------------------------------
+def raw2alpha(sigma, dist):
+    """app/tools/utils.py:51-64. Returns (alpha, weights, T_last)."""
+    alpha = 1.0 - torch.exp(-sigma * dist)
+    T = torch.cumprod(
+        torch.cat([torch.ones(alpha.shape[0], 1, device=alpha.device), 1.0 - alpha + 1e-10], -1), -1
+    )
+    return alpha, alpha * T[:, :-1], T[:, -1:]
+
+
+# --------------------------------------------------------------------------------------
+# colour network
+# --------------------------------------------------------------------------------------
+def positional_encoding(x, freqs):
+    """app/tools/utils.py:42-48."""
+    bands = 2 ** torch.arange(freqs, dtype=torch.float, device=x.device)
+    q = (x[..., None] * bands).reshape(x.shape[:-1] + (freqs * x.shape[-1],))
+    return torch.cat([torch.sin(q), torch.cos(q)], dim=-1)
+
+
+def mlp_input(p, viewdirs, feats):
+    """Row layout of the network input, app/models/mlp_render_fea.py:55-65
+    (encode_app off): [feat | view | PE(feat) | PE(view)]."""
+    parts = [feats]
+    if p.view_pe > -1:
+        parts.append(viewdirs)
+    if p.fea_pe > 0:
+        parts.append(positional_encoding(feats, p.fea_pe))
+    if p.view_pe > 0:
+        parts.append(positional_encoding(viewdirs, p.view_pe))
+    return torch.cat(parts, dim=-1)
+
+
+def mlp_render(p, viewdirs, feats):
+    """app/models/mlp_render_fea.py:30-41,66-68: Linear-ReLU-Linear-ReLU-Linear-sigmoid."""
+    h = mlp_input(p, viewdirs, feats)
+    h = F.relu(F.linear(h, p.mlp_w[0], p.mlp_b[0]))
+    h = F.relu(F.linear(h, p.mlp_w[1], p.mlp_b[1]))
+    h = F.linear(h, p.mlp_w[2], p.mlp_b[2])
+    return torch.sigmoid(h)
+
+
+# --------------------------------------------------------------------------------------
+# whole chunk
+# --------------------------------------------------------------------------------------
+@torch.no_grad()
+def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False):
+    """GridBaseSequential.forward with is_train=False,
+    app/models/gridnerf_sequential.py:448-504 (sampling_opt=0) and :523-576
+    (sampling_opt=1); the two branches differ only in the sampler."""
+    rays_o = rays_chunk[:, :3]
+    rays_d = viewdirs = rays_chunk[:, 3:6]
+    if p.sampling_opt:
+        xyz, z, ray_valid = sample_ray_within_hull(p, rays_o, viewdirs, p.n_importance)
+    else:
+        xyz, z, ray_valid = sample_ray_aabb(p, rays_o, viewdirs, N_samples)
+    dists = torch.cat((z[:, 1:] - z[:, :-1], torch.zeros_like(z[:, :1])), dim=-1)
+    viewdirs = viewdirs.view(-1, 1, 3).expand(xyz.shape)
+
+    if p.alpha_volume is not None:
+        alphas = sample_alpha(p.alpha_volume, p.alpha_aabb, xyz[ray_valid])
+        keep = alphas > p.alpha_mask_filter_thre
+        ray_invalid = ~ray_valid
+        ray_invalid[ray_valid] |= ~keep
+        ray_valid = ~ray_invalid
+
+    sigma = torch.zeros(xyz.shape[:-1], device=xyz.device)
+    rgb = torch.zeros((*xyz.shape[:2], 3), device=xyz.device)
+    if ray_valid.any():
+        xyz = normalize_coord(p, xyz)
+        sigma[ray_valid] = feature2density(p, density_feature(p, xyz[ray_valid]))
+
+    _, weight, _ = raw2alpha(sigma, dists * p.distance_scale)
+    app_mask = weight > p.rayMarch_weight_thres
+    if app_mask.any():
+        feats = app_feature(p, xyz[app_mask])
+        rgb[app_mask] = mlp_render(p, viewdirs[app_mask], feats)
+
+    acc = torch.sum(weight, -1)
+    rgb_map = torch.sum(weight[..., None] * rgb, -2)
+    if white_bg:
+        rgb_map = rgb_map + (1.0 - acc[..., None])
+    rgb_map = rgb_map.clamp(0, 1)
+    depth_map = torch.sum(weight * z, -1)
+    out = {"rgb_map": rgb_map, "depth_map": depth_map}
+    if return_aux:
+        out.update(
+            {
+                "ray_valid": ray_valid,
+                "z_vals": z,
+                "sigma": sigma,
+                "weight": weight,
+                "app_mask": app_mask,
+                "acc_map": acc,
+                "rgb": rgb,
+            }
+        )
+    return out
+
+
+def renderer_fn(
+    rays, model, chunk=4096, N_samples=-1, white_bg=True, is_train=False, device="cpu", idxs=None
+) -> Tuple[Dict[str, torch.Tensor], dict]:
+    """Chunk loop, app/tools/render_utils.py:15-63, driving `render_chunk` on `model`
+    (a parameter object).  `is_train` and `idxs` are accepted and must be off."""
+    assert not is_train and idxs is None
+    acc: Dict[str, list] = {}
+    n = rays.shape[0]
+    for i in range(n // chunk + int(n % chunk > 0)):
+        ret = render_chunk(model, rays[i * chunk : (i + 1) * chunk].to(device), white_bg=white_bg, N_samples=N_samples)
+        for k, v in ret.items():
+            acc.setdefault(k, []).append(v)
+    return {k: torch.cat(v, 0) for k, v in acc.items()}, {}
+
+
+def to_fp16_features(p):
+    """Parameter object with planes and lines stored in fp16 (interpolated in fp32)."""
+    import copy
+
+    q = copy.copy(p)
+    q.density_plane = [t.half() for t in p.density_plane]
+    q.density_line = [t.half() for t in p.density_line]
+    q.app_plane = [t.half() for t in p.app_plane]
+    q.app_line = [t.half() for t in p.app_line]
+    return q

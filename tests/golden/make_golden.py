@@ -1,0 +1,197 @@
+"""Write the golden vectors in this directory from the reference's own forward.
+
+Run once, in the build container only (needs the reference checkout, default
+/root/reference):  python tests/golden/make_golden.py
+
+What it pins.  Every arithmetic piece of the render path reduces to a PyTorch
+library routine and is checked against closed forms and brute force elsewhere in
+tests/.  What those checks cannot see is the *composition* inside
+GridBaseSequential.forward (app/models/gridnerf_sequential.py:439-658): occupancy
+lookup on un-normalised points, the ray_valid update idiom, the zero last interval,
+the 1e-10 inside the cumulative product, the mask on weights rather than alpha, white
+background before the clamp, unclamped depth, the plane index -> (dimension, level)
+mapping, and the colour network's input order.  So this script builds the reference
+model on the CPU, runs `forward(is_train=False)` and the sub-functions it calls on
+small seeded inputs, and stores inputs, parameters and outputs as .npz data.
+
+The reference's module top levels import packages that are absent here and that the
+render branch never calls (torch_efficient_distloss, cv2, kornia, and the dataset /
+parallel-model modules pulled in by two package __init__ files).  They are replaced
+by empty stand-ins in sys.modules; no reference code is modified or copied.
+"""
+import os
+import sys
+import types
+from types import SimpleNamespace
+
+import numpy as np
+import torch
+
+REF = os.environ.get("LANDMARK_REFERENCE", "/root/reference")
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _install_stand_ins():
+    def pkg(name, path):
+        m = types.ModuleType(name)
+        m.__path__ = [path]
+        sys.modules[name] = m
+        return m
+
+    # packages whose __init__ would import datasets / parallel model variants
+    pkg("app", os.path.join(REF, "app"))
+    pkg("app.tools", os.path.join(REF, "app", "tools"))
+    pkg("app.tools.dataloader", os.path.join(REF, "app", "tools", "dataloader"))
+    pkg("app.models", os.path.join(REF, "app", "models"))
+    # third-party modules absent from this image, unused by the render branch
+    dl = types.ModuleType("torch_efficient_distloss")
+    dl.eff_distloss = lambda *a, **k: (_ for _ in ()).throw(RuntimeError("training only"))
+    sys.modules["torch_efficient_distloss"] = dl
+    cv2 = types.ModuleType("cv2")
+    cv2.COLORMAP_JET = 2
+    sys.modules["cv2"] = cv2
+    kornia = types.ModuleType("kornia")
+    kornia.create_meshgrid = lambda *a, **k: (_ for _ in ()).throw(RuntimeError("unused"))
+    sys.modules["kornia"] = kornia
+
+
+def _args(**kw):
+    base = dict(
+        distributed=False,
+        run_nerf=False,
+        nonlinear_density=False,
+        ndims=3,
+        TV_weight_density=0,
+        TV_weight_app=0,
+        resMode=[1],
+        sampling_opt=1,
+        bias_enable=1,
+        encode_app=False,
+        n_importance=16,
+        alpha_mask_filter_thre=0.0,
+        ckpt=None,
+        device="cpu",
+    )
+    base.update(kw)
+    return SimpleNamespace(**base)
+
+
+def _camera_rays(n_side, eye, seed):
+    """Small pinhole fan above the scene looking down-ish (blender convention)."""
+    g = torch.Generator().manual_seed(seed)
+    eye = torch.tensor(eye, dtype=torch.float32)
+    fwd = -eye / eye.norm()
+    right = torch.linalg.cross(fwd, torch.tensor([0.0, 0.0, 1.0]))
+    right = right / right.norm()
+    up = torch.linalg.cross(right, fwd)
+    u = torch.linspace(-0.45, 0.45, n_side)
+    jj, ii = torch.meshgrid(u, u, indexing="ij")
+    d = ii[..., None] * right - jj[..., None] * up + fwd
+    d = d.reshape(-1, 3) + 0.01 * torch.randn(n_side * n_side, 3, generator=g)
+    o = eye.expand_as(d)
+    return torch.cat([o, d], 1).contiguous()
+
+
+def _generic_rays(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    o = torch.randn(n, 3, generator=g) * 0.4 + torch.tensor([0.0, 0.0, 1.6])
+    d = torch.randn(n, 3, generator=g)
+    d[:, 2] = -d[:, 2].abs() - 0.2
+    d[0, 0] = 0.0  # exercise the zero-component guard of the slab test
+    d[1, 1] = 0.0
+    o[2] = torch.tensor([5.0, 5.0, 5.0])  # a ray that misses the box
+    d[3, 2] = 0.3  # upward ray
+    return torch.cat([o, d], 1).contiguous()
+
+
+CASES = [
+    # name, model kwargs, args kwargs, extras
+    dict(name="hull_softplus_L1", grid=[6, 7, 5], dn=16, an=48, act="softplus", shift=0.0, res=[1], ndims=3, opt=1, mask=True, thre=0.0, S=16, boost=8.0),
+    dict(name="hull_relu_L2", grid=[6, 7, 5], dn=16, an=48, act="relu", shift=-10.0, res=[1, 2], ndims=3, opt=1, mask=True, thre=0.5, S=16, boost=12.0),
+    dict(name="hull_relu_L3_P1", grid=[5, 6, 4], dn=16, an=48, act="relu", shift=-10.0, res=[1, 2, 4], ndims=1, opt=1, mask=False, thre=0.0, S=24, boost=20.0),
+    dict(name="aabb_softplus_L1", grid=[6, 7, 5], dn=16, an=48, act="softplus", shift=-1.0, res=[1], ndims=3, opt=0, mask=True, thre=0.0, S=20, boost=10.0, sr=0.25),
+    dict(name="aabb_relu_L2_nomask", grid=[4, 5, 6], dn=8, an=12, act="relu", shift=-10.0, res=[1, 2], ndims=2, opt=0, mask=False, thre=0.0, S=-1, boost=15.0, sr=0.5),
+    dict(name="hull_softplus_trivial", grid=[6, 7, 5], dn=16, an=48, act="softplus", shift=-10.0, res=[1], ndims=3, opt=1, mask=False, thre=0.0, S=16, boost=1.0),
+]
+
+
+def main():
+    if not os.path.isdir(REF):
+        raise SystemExit(f"reference checkout not found at {REF}")
+    _install_stand_ins()
+    sys.path.insert(0, REF)
+    from app.models.alpha_mask import AlphaGridMask  # noqa: E402
+    from app.models.gridnerf_sequential import GridNeRF  # noqa: E402
+    from app.tools.utils import positional_encoding, raw2alpha  # noqa: E402
+
+    for ci, c in enumerate(CASES):
+        torch.manual_seed(100 + ci)
+        aabb = torch.tensor([[-1.0, -1.2, -0.8], [1.1, 1.0, 0.9]])
+        args = _args(
+            ndims=c["ndims"], resMode=c["res"], sampling_opt=c["opt"], n_importance=max(c["S"], 8),
+            alpha_mask_filter_thre=c["thre"],
+        )
+        model = GridNeRF(
+            aabb, c["grid"], "cpu",
+            density_n_comp=[c["dn"]] * 3, appearance_n_comp=[c["an"]] * 3, app_dim=27,
+            near_far=[0.4, 4.0], density_shift=c["shift"], distance_scale=25, rayMarch_weight_thres=0.001,
+            pos_pe=2, view_pe=2, fea_pe=2, featureC=128, step_ratio=c.get("sr", 2.0),
+            fea2denseAct=c["act"], args=args, is_train=False,
+        )
+        model.eval()
+        with torch.no_grad():
+            for t in model.density_plane:
+                t.mul_(c["boost"])
+            if c["mask"]:
+                g = torch.Generator().manual_seed(7 + ci)
+                vol = (torch.rand(5, 7, 6, generator=g) < 0.6).float()
+                mask_aabb = aabb + torch.tensor([[0.05, -0.02, 0.0], [0.0, 0.03, -0.04]])
+                model.alphaMask = AlphaGridMask("cpu", mask_aabb, vol)
+            rays = _camera_rays(7, (1.4, -1.1, 1.9), 11 + ci) if c["opt"] else _generic_rays(40, 11 + ci)
+            (out, extra) = model(rays, is_train=False, white_bg=True, N_samples=c["S"])
+            (out_black, _) = model(rays, is_train=False, white_bg=False, N_samples=c["S"])
+            # sub-function vectors on the same model
+            if c["opt"]:
+                pts, _, z, inside = model.sample_ray_within_hull(rays[:, :3], rays[:, 3:6], is_train=False, N_samples=model.n_importance)
+            else:
+                pts, _, z, inside = model.sample_ray(rays[:, :3], rays[:, 3:6], is_train=False, N_samples=c["S"])
+            q = model.normalize_coord(pts).reshape(-1, 3)
+            dens = model.compute_densityfeature(q)
+            appf = model.compute_appfeature(q)
+            vd = rays[:, None, 3:6].expand(pts.shape).reshape(-1, 3)
+            rgb = model.renderModule(vd, appf)
+            sig = model.feature2density(dens)
+            dists = torch.cat((z[:, 1:] - z[:, :-1], torch.zeros_like(z[:, :1])), dim=-1)
+            alpha, weight, t_last = raw2alpha(sig.view(z.shape), dists * model.distance_scale)
+            pe = positional_encoding(appf[:5], 2)
+            store = {
+                "rays": rays, "rgb_map": out["rgb_map"], "depth_map": out["depth_map"],
+                "rgb_map_black": out_black["rgb_map"],
+                "sub_pts": pts, "sub_z": z, "sub_inside": inside, "sub_density_feature": dens,
+                "sub_app_feature": appf, "sub_rgb": rgb, "sub_alpha": alpha, "sub_weight": weight,
+                "sub_t_last": t_last, "sub_pe": pe, "aabb": aabb,
+            }
+            if c["mask"]:
+                store["alpha_volume"] = model.alphaMask.alpha_volume[0, 0]
+                store["alpha_aabb"] = model.alphaMask.aabb
+                store["sub_alpha_lookup"] = model.alphaMask.sample_alpha(pts.reshape(-1, 3))
+            for k, v in model.state_dict().items():
+                store["sd." + k] = v
+            assert extra == {}
+        cfg = dict(
+            grid=c["grid"], ndims=c["ndims"], resMode=c["res"], sampling_opt=c["opt"], N_samples=c["S"],
+            n_importance=int(model.n_importance), near_far=[0.4, 4.0], density_shift=c["shift"],
+            fea2denseAct=c["act"], step_ratio=float(model.step_ratio), thre=c["thre"], nSamples=int(model.nSamples),
+            stepSize=float(model.stepSize),
+        )
+        arrays = {k: (v.detach().cpu().numpy() if torch.is_tensor(v) else np.asarray(v)) for k, v in store.items()}
+        arrays["cfg_json"] = np.frombuffer(__import__("json").dumps(cfg).encode(), dtype=np.uint8)
+        path = os.path.join(HERE, f"forward_{c['name']}.npz")
+        np.savez_compressed(path, **arrays)
+        n_app = int((weight > 0.001).sum())
+        print(f"{c['name']}: rays {tuple(rays.shape)} S={z.shape[1]} valid-in-box {int(inside.sum())} "
+              f"weights>thr {n_app} rgb mean {out['rgb_map'].mean():.4f} -> {os.path.getsize(path)/1024:.0f} KB")
+
+
+if __name__ == "__main__":
+    main()

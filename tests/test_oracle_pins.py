@@ -1,0 +1,231 @@
+"""Pins for the PyTorch oracle that do not come from the reference: a from-scratch
+scalar C restatement (oracle/scalar_ref.c), closed forms and brute force.  Each check
+is chosen so that a plausible slip (dropped term, swapped axis, wrong index order,
+fused multiply-add) fails it."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from landmark_amd import scenes
+from oracle import gridnerf_oracle as O
+from oracle import scalar_ref as SR
+from tests.helpers import golden_names, load_golden
+
+
+# ---------------------------------------------------------------- scalar C vs torch, whole path
+@pytest.mark.parametrize("name", golden_names())
+def test_scalar_restatement_matches_oracle(name):
+    p, d, cfg = load_golden(name)
+    sm = SR.ScalarModel(p, N_samples=cfg["N_samples"])
+    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], return_aux=True)
+    valid, z, cnt = sm.sample_cull(d["rays"])
+    assert torch.equal(z, ref["z_vals"]), "z values must be bit-identical"
+    assert torch.equal(valid, ref["ray_valid"]), "sample mask must be bit-identical"
+    assert cnt == int(ref["ray_valid"].sum())
+    out = sm.render(d["rays"])
+    assert torch.equal(out["ray_valid"], ref["ray_valid"])
+    assert torch.allclose(out["sigma"], ref["sigma"], atol=2e-5, rtol=1e-5)
+    assert torch.allclose(out["weight"], ref["weight"], atol=1e-5)
+    near_thr = (ref["weight"] - p.rayMarch_weight_thres).abs() < 1e-6
+    assert torch.equal(out["app_mask"] | near_thr, ref["app_mask"] | near_thr)
+    assert torch.allclose(out["rgb_map"], ref["rgb_map"], atol=2e-5)
+    assert torch.allclose(out["depth_map"], ref["depth_map"], atol=2e-5)
+
+
+def test_scalar_mask_bit_exact_on_larger_random_scene():
+    p = scenes.make_params(seed=3, gridSize=(9, 11, 13), near_far=[0.5, 4.5], n_importance=64, sampling_opt=1)
+    p.alpha_volume = scenes.blob_occupancy((9, 11, 13), 6, 0.4, seed=1)
+    p.alpha_aabb = p.aabb + torch.tensor([[0.01, 0.0, -0.02], [0.0, 0.05, 0.0]])
+    rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    for thre in (0.0, 0.5, 0.98):
+        p.alpha_mask_filter_thre = thre
+        ref = O.render_chunk(p, rays, return_aux=True)
+        valid, z, _ = SR.ScalarModel(p).sample_cull(rays)
+        assert torch.equal(valid, ref["ray_valid"]) and torch.equal(z, ref["z_vals"])
+        assert 0 < int(valid.sum()) < valid.numel()
+    p.sampling_opt = 0
+    p.step_ratio = 0.4
+    ref = O.render_chunk(p, rays, N_samples=50, return_aux=True)
+    valid, z, _ = SR.ScalarModel(p, N_samples=50).sample_cull(rays)
+    assert torch.equal(valid, ref["ray_valid"]) and torch.equal(z, ref["z_vals"])
+
+
+# ---------------------------------------------------------------- sampling closed forms
+def _geom_params(**kw):
+    return scenes.make_params(seed=0, gridSize=(5, 5, 5), density_n_comp=4, app_n_comp=4, **kw)
+
+
+def test_hull_sampler_closed_forms():
+    p = _geom_params(near_far=[0.5, 4.5], sampling_opt=1)
+    o = torch.tensor([[0.0, 0.0, 2.0], [0.3, -0.2, 1.5], [0.0, 0.0, 2.0]])
+    d = torch.tensor([[0.0, 0.0, -1.0], [0.1, 0.2, -0.5], [0.0, 0.1, 0.4]])
+    pts, z, inside = O.sample_ray_within_hull(p, o, d, 33)
+    assert torch.all(z[:, 0] == 0.5)
+    # downward rays end exactly on the floor z = aabb_min_z
+    assert z[0, -1].item() == pytest.approx(3.0) and z[1, -1].item() == pytest.approx(5.0)
+    assert torch.allclose(pts[:2, -1, 2], torch.tensor([-1.0, -1.0]), atol=1e-6)
+    assert z[2, -1].item() == 4.5  # upward ray: far plane
+    assert torch.all(z[:, 1:] > z[:, :-1])
+    # vertical ray through the box centre: inside iff -1 <= 2 - z <= 1
+    exp_inside = (2.0 - z[0] >= -1.0) & (2.0 - z[0] <= 1.0)
+    assert torch.equal(inside[0], exp_inside)
+
+
+def test_aabb_sampler_closed_forms():
+    p = _geom_params(near_far=[0.1, 6.0], sampling_opt=0, step_ratio=0.5)
+    step = float(p.stepSize)
+    assert step == pytest.approx(0.5 * 0.5)  # aabb size 2 / (5-1) * ratio
+    o = torch.tensor([[-3.0, 0.0, 0.0], [0.0, 0.0, 0.0], [0.0, 5.0, 0.0], [-3.0, 0.5, 0.0]])
+    d = torch.tensor([[1.0, 0.0, 0.0], [0.0, 1.0, 0.0], [0.0, -2.0, 0.0], [1.0, 0.0, 0.0]])
+    pts, z, inside = O.sample_ray_aabb(p, o, d, 12)
+    assert z[0, 0].item() == pytest.approx(2.0)  # enters x=-1 at t=2
+    assert z[1, 0].item() == pytest.approx(0.1)  # origin inside the box: clamped to near
+    assert z[2, 0].item() == pytest.approx(2.0)  # |d|=2: enters y=1 at t=2
+    assert torch.allclose(z[:, 1:] - z[:, :-1], torch.full((4, 11), step))
+    assert inside[0, 0] and inside[0, 8] and not inside[0, 9]  # 2 + 9*0.25 > 3
+    assert p.nSamples == int(math.sqrt(12.0) / step) + 1
+
+
+# ---------------------------------------------------------------- occupancy invariants
+def test_alpha_lookup_invariants_and_scalar_loop():
+    aabb = torch.tensor([[-1.0, -2.0, 0.0], [1.0, 2.0, 3.0]])
+    g = torch.Generator().manual_seed(0)
+    pts = torch.rand(500, 3, generator=g) * (aabb[1] - aabb[0]) + aabb[0]
+    ones = torch.ones(4, 5, 6)
+    assert torch.all(O.sample_alpha(ones, aabb, pts) > 0.999)
+    assert torch.all(O.sample_alpha(torch.zeros(4, 5, 6), aabb, pts) == 0)
+    # a single voxel: non-zero exactly within one cell of it along every axis
+    vol = torch.zeros(4, 5, 6)
+    vol[2, 1, 3] = 1.0  # z index 2, y index 1, x index 3
+    val = O.sample_alpha(vol, aabb, pts)
+    ix = (pts[:, 0] - aabb[0, 0]) / (aabb[1, 0] - aabb[0, 0]) * 5
+    iy = (pts[:, 1] - aabb[0, 1]) / (aabb[1, 1] - aabb[0, 1]) * 4
+    iz = (pts[:, 2] - aabb[0, 2]) / (aabb[1, 2] - aabb[0, 2]) * 3
+    expect = (1 - (ix - 3).abs()).clamp(min=0) * (1 - (iy - 1).abs()).clamp(min=0) * (1 - (iz - 2).abs()).clamp(min=0)
+    assert torch.allclose(val, expect, atol=1e-5)
+    # voxel centres reproduce the voxel values; axis order x->W, y->H, z->D
+    rnd = torch.rand(4, 5, 6, generator=g)
+    zz, yy, xx = torch.meshgrid(torch.arange(4), torch.arange(5), torch.arange(6), indexing="ij")
+    centres = torch.stack([xx / 5 * 2 - 1, yy / 4 * 4 - 2, zz / 3 * 3.0], -1).reshape(-1, 3).float()
+    assert torch.allclose(O.sample_alpha(rnd, aabb, centres), rnd.reshape(-1), atol=1e-6)
+
+
+# ---------------------------------------------------------------- plane / line lookup
+def test_feature_lookup_affine_and_texel_centres():
+    p = scenes.make_params(seed=1, gridSize=(7, 5, 9), density_n_comp=2, app_n_comp=4, ndims=3, resMode=(1, 2))
+    # make every density plane affine in its own (x, y) and every line constant 1:
+    L = 2
+    coef = []
+    for k, pl in enumerate(p.density_plane):
+        H, W = pl.shape[-2:]
+        ys, xs = torch.meshgrid(torch.linspace(-1, 1, H), torch.linspace(-1, 1, W), indexing="ij")
+        a, b, c = 0.3 + 0.1 * k, -0.2 + 0.05 * k, 0.7 - 0.02 * k
+        pl[0, 0] = a * xs + b * ys + c
+        pl[0, 1] = 0
+        p.density_line[k].fill_(1.0)
+        coef.append((a, b, c))
+    g = torch.Generator().manual_seed(2)
+    xyz = torch.rand(300, 3, generator=g) * 2 - 1
+    got = O.density_feature(p, xyz)
+    exp = torch.zeros(300)
+    for k, (a, b, c) in enumerate(coef):
+        m0, m1 = O.MAT_MODE[k // L]
+        exp += a * xyz[:, m0] + b * xyz[:, m1] + c  # bilinear reproduces affine functions
+    assert torch.allclose(got, exp, atol=1e-5)
+
+
+def test_line_uses_vec_mode_axis_and_product_columns():
+    p = scenes.make_params(seed=2, gridSize=(4, 5, 6), density_n_comp=2, app_n_comp=3, ndims=3, resMode=(1, 2))
+    L, Ca = 2, 3
+    for k in range(6):
+        p.app_plane[k].fill_(1.0)
+        Len = p.app_line[k].shape[2]
+        ramp = torch.linspace(-1, 1, Len)
+        for c in range(Ca):
+            p.app_line[k][0, c, :, 0] = (k * 10 + c) + ramp  # linear interp reproduces a ramp exactly
+    xyz = torch.tensor([[0.31, -0.52, 0.77], [-0.9, 0.4, 0.05]])
+    prod = O.app_products(p, xyz)
+    assert prod.shape == (2, 18)
+    for k in range(6):
+        axis = O.VEC_MODE[k // L]
+        for c in range(Ca):
+            assert torch.allclose(prod[:, k * Ca + c], (k * 10 + c) + xyz[:, axis], atol=1e-5)
+    # basis_mat is a plain matmul over those columns (one-hot probe)
+    p.basis_mat = torch.zeros(27, 18)
+    p.basis_mat[5, 2 * Ca + 1] = 1.0
+    f = O.app_feature(p, xyz)
+    assert torch.allclose(f[:, 5], prod[:, 2 * Ca + 1]) and f[:, :5].abs().sum() == 0
+
+
+def test_bilinear_against_scalar_loop_with_padding():
+    g = torch.Generator().manual_seed(3)
+    img = torch.randn(1, 1, 4, 5, generator=g)
+    pts = torch.rand(400, 2, generator=g) * 2.4 - 1.2  # includes points outside [-1,1]
+    got = F.grid_sample(img, pts.view(1, -1, 1, 2), align_corners=True).view(-1)
+    lib = SR.lib()
+    arr = np.ascontiguousarray(img[0, 0].numpy())
+    import ctypes as C
+
+    exp = [lib.lmref_bilinear(arr.ctypes.data_as(C.POINTER(C.c_float)), 4, 5, C.c_float(x), C.c_float(y)) for x, y in pts.tolist()]
+    assert torch.allclose(got, torch.tensor(exp), atol=1e-6)
+
+
+# ---------------------------------------------------------------- compositing
+def test_raw2alpha_double_loop_and_identities():
+    g = torch.Generator().manual_seed(4)
+    sigma = torch.rand(6, 9, generator=g) * 3
+    sigma[0] = 0
+    sigma[1, 0] = 1e4
+    dist = torch.rand(6, 9, generator=g) * 0.5
+    dist[:, -1] = 0
+    a, w, t = O.raw2alpha(sigma, dist)
+    for r in range(6):
+        T = 1.0
+        for s in range(9):
+            al = 1.0 - math.exp(-float(sigma[r, s]) * float(dist[r, s]))
+            assert float(w[r, s]) == pytest.approx(al * T, abs=1e-6)
+            T *= 1.0 - al + 1e-10
+        assert float(t[r, 0]) == pytest.approx(T, abs=1e-6)
+    assert torch.all(w[0] == 0) and torch.all(w[:, -1] == 0)  # sigma=0 ; last interval is zero
+    assert float(w[1, 0]) == pytest.approx(1.0, abs=1e-6) and float(w[1, 1:].sum()) < 1e-6
+    assert torch.allclose(w.sum(-1), 1 - t[:, 0], atol=1e-5)
+    c = 0.7  # constant sigma, constant step: w_i = (1-e)^... closed form
+    w2 = O.raw2alpha(torch.full((1, 5), c), torch.full((1, 5), 0.2))[1][0]
+    e = math.exp(-c * 0.2)
+    assert torch.allclose(w2, torch.tensor([(1 - e) * e**i for i in range(5)]), atol=1e-6)
+
+
+# ---------------------------------------------------------------- colour network
+def test_positional_encoding_order_and_values():
+    x = torch.tensor([[0.3, -1.2, 2.0]])
+    pe = O.positional_encoding(x, 2)[0]
+    exp = [math.sin(v * f) for v in (0.3, -1.2, 2.0) for f in (1, 2)] + [math.cos(v * f) for v in (0.3, -1.2, 2.0) for f in (1, 2)]
+    assert torch.allclose(pe, torch.tensor(exp), atol=1e-6)
+
+
+def test_mlp_against_float64_and_input_layout():
+    p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=2, app_n_comp=2)
+    g = torch.Generator().manual_seed(6)
+    feats, view = torch.randn(50, 27, generator=g), torch.randn(50, 3, generator=g)
+    x = O.mlp_input(p, view, feats)
+    assert x.shape == (50, 150)
+    assert torch.equal(x[:, :27], feats) and torch.equal(x[:, 27:30], view)
+    assert torch.allclose(x[:, 30], torch.sin(feats[:, 0])) and torch.allclose(x[:, 31], torch.sin(2 * feats[:, 0]))
+    assert torch.allclose(x[:, 84], torch.cos(feats[:, 0])) and torch.allclose(x[:, 138], torch.sin(view[:, 0]))
+    assert torch.allclose(x[:, 149], torch.cos(2 * view[:, 2]))
+    h = x.double().numpy()
+    for i in range(3):
+        h = h @ p.mlp_w[i].double().numpy().T + p.mlp_b[i].double().numpy()
+        if i < 2:
+            h = np.maximum(h, 0)
+    exp = 1 / (1 + np.exp(-h))
+    assert np.allclose(O.mlp_render(p, view, feats).numpy(), exp, atol=1e-5)
+
+
+def test_normalize_coord_maps_corners():
+    p = scenes.make_params(seed=0, aabb=((-3, -3, -0.1), (3, 3, 1)), gridSize=(4, 4, 4), density_n_comp=2, app_n_comp=2)
+    assert torch.equal(O.normalize_coord(p, p.aabb[0][None]), -torch.ones(1, 3))
+    assert torch.allclose(O.normalize_coord(p, p.aabb[1][None]), torch.ones(1, 3), atol=1e-6)
