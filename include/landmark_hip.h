@@ -1,0 +1,200 @@
+/* landmark_hip.h -- C ABI of the MI355X (gfx950) GridNeRF render path.
+ *
+ * Drop-in boundary for the single-GPU render branch of InternLandMark/LandMark.  Every
+ * entry point names the reference interface it replaces (paths relative to the
+ * reference checkout).  Conventions:
+ *   - plain pointers and sizes; all array pointers are DEVICE pointers unless the
+ *     parameter is documented as host memory; device pointers must be 16-byte aligned;
+ *   - the caller owns every buffer (inputs, outputs and the workspace); the library
+ *     allocates nothing and keeps no global state besides a thread-local error string;
+ *   - every function takes the HIP stream to launch on (`void*` = hipStream_t, NULL =
+ *     the null stream) and returns without waiting for the GPU;
+ *   - return value: LM_OK (0) or a negative lm_status; lm_last_error() describes the
+ *     last failure on the calling thread.  Nothing here calls exit() or abort().
+ *
+ * Data layout.  Feature planes are channel-last: plane[H][W][C] and line[Len][C]
+ * (the reference stores [1,C,H,W] and [1,C,Len,1]; lm_relayout_nchw_to_hwc converts).
+ * Samples are addressed by their flat index ray*S + s.  The valid-sample list is the
+ * ascending list of flat indices that pass the AABB and occupancy tests: the same
+ * order the reference's boolean-mask indexing produces.
+ */
+#ifndef LANDMARK_HIP_H
+#define LANDMARK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LM_ABI_VERSION 1
+#define LM_MAX_PLANES 12 /* ndims * len(resMode) */
+
+typedef enum lm_status {
+    LM_OK = 0,
+    LM_ERR_INVALID = -1,     /* bad argument (null, misaligned, out of range) */
+    LM_ERR_UNSUPPORTED = -2, /* valid in the reference, not implemented here */
+    LM_ERR_LAUNCH = -3,      /* HIP reported an error at launch */
+    LM_ERR_WORKSPACE = -4    /* workspace too small */
+} lm_status;
+
+enum { LM_F32 = 0, LM_F16 = 1 };                   /* plane / line storage type */
+enum { LM_SAMPLER_AABB = 0, LM_SAMPLER_HULL = 1 }; /* sampling_opt 0 / 1 */
+enum { LM_ACT_SOFTPLUS = 0, LM_ACT_RELU = 1 };     /* fea2denseAct */
+/* arithmetic of the colour network's matrix products (accumulation is always fp32) */
+enum { LM_MLP_F32 = 0, LM_MLP_F16 = 1, LM_MLP_BF16 = 2 };
+
+/* One feature plane with its line (one entry of density_plane/density_line or
+ * app_plane/app_line, app/models/gridnerf_sequential.py:676-718).  ax0/ax1 select the
+ * normalised coordinates used as the plane's x (-> W) and y (-> H), axl the line's
+ * (matMode / vecMode, gridnerf_sequential.py:106-107). */
+typedef struct lm_plane {
+    const void *plane; /* [H][W][C] */
+    const void *line;  /* [Len][C]  */
+    int32_t H, W, Len, C;
+    int32_t ax0, ax1, axl;
+    int32_t dtype; /* LM_F32 | LM_F16 */
+} lm_plane;
+
+/* Ray sampling and occupancy culling parameters.
+ * sampler HULL (gridnerf_sequential.py:298-319): z = tab_a[s] + far_ray * tab_t[s] with
+ *   tab_t = torch.linspace(0,1,S), tab_a = near*(1-tab_t), far_ray = -((o_z-aabb_min_z)/d_z)
+ *   or `far` when d_z >= 0.
+ * sampler AABB (gridnerf_sequential.py:260-281): z = t_min + tab_a[s] with
+ *   tab_a = stepSize*arange(S), t_min = slab entry clamped to [near, far].
+ * The tables are passed in (device memory) because torch.linspace is not reproducible
+ * from i/(S-1) in float arithmetic.  inv_aabb = 2/aabbSize and vol_inv = 1/size*2 are
+ * computed by the caller in float exactly as the reference does
+ * (gridnerf_sequential.py:158-159, alpha_mask.py:20-22). */
+typedef struct lm_geom {
+    int32_t sampler;
+    int32_t S;
+    float aabb[6]; /* min xyz, max xyz */
+    float near_, far_;
+    const float *tab_a; /* [S] */
+    const float *tab_t; /* [S] */
+    float inv_aabb[3];
+    /* occupancy volume (app/models/alpha_mask.py); vol == NULL: no culling */
+    const float *vol; /* [vd][vh][vw] */
+    int32_t vd, vh, vw;
+    float vol_aabb_min[3];
+    float vol_inv[3];
+    float vol_thre; /* alpha_mask_filter_thre */
+} lm_geom;
+
+typedef struct lm_model {
+    lm_geom geom;
+    int32_t n_planes; /* ndims * levels, plane index k = dim * levels + level */
+    lm_plane density[LM_MAX_PLANES];
+    lm_plane app[LM_MAX_PLANES];
+    int32_t act;         /* LM_ACT_* */
+    float density_shift; /* softplus(f + shift) */
+    float distance_scale;
+    float weight_thres; /* rayMarch_weight_thres */
+    int32_t mlp_prec;   /* LM_MLP_* the packed weights were packed for */
+    const void *mlp_packed; /* device copy of the buffer written by lm_mlp_pack */
+    int32_t white_bg;
+    float term_eps; /* > 0: stop marching a ray once transmittance < term_eps */
+} lm_model;
+
+/* Counters written by lm_render (device memory, 8 x uint32). */
+enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_WORDS = 8 };
+
+int lm_abi_version(void);
+const char *lm_last_error(void);
+
+/* [C,H,W] -> [H,W,C] (and [C,Len] -> [Len,C] with W = 1).  The reference keeps NCHW
+ * parameters (gridnerf_sequential.py:703-718); its dynamic-fetching variant re-lays them
+ * out channel-last the same way (app/models/gridnerf_elastic_cuda.py:274-303). */
+int lm_relayout_nchw_to_hwc(const void *src, void *dst, int32_t C, int32_t H, int32_t W, int32_t dtype,
+                            void *stream);
+
+/* ---- part 1: sampling + AABB / occupancy culling + stable compaction -----------------
+ * Replaces sample_ray / sample_ray_within_hull + AlphaGridMask.sample_alpha + the
+ * boolean-mask indexing of GridBaseSequential.forward
+ * (gridnerf_sequential.py:244-319, 453-465, 528-541; alpha_mask.py:35-59); prior art
+ * SamplerayGridsample.cuda (dist_render/kernel/cuda_kernel/sampleray_gridsample/
+ * compute_sampleray_gridsample_cuda.cpp:34-151).
+ *   rays        [N,6]  origin, direction
+ *   bitmap      [ceil(N*S/64)] uint64, bit (i & 63) of word i>>6 = sample i is valid
+ *   word_prefix [ceil(N*S/64)] uint32, number of valid samples before each word
+ *   valid_idx   [N*S] uint32 capacity, ascending flat indices of valid samples
+ *   counters    [LM_STAT_WORDS] uint32, counters[LM_STAT_N_VALID] = number of valid samples
+ *   z_out       optional [N*S] sample depths (NULL to skip)
+ *   scratch     lm_sample_cull_scratch_bytes(N,S) bytes
+ */
+size_t lm_sample_cull_scratch_bytes(int64_t N, int32_t S);
+int lm_sample_cull(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *word_prefix,
+                   uint32_t *valid_idx, uint32_t *counters, float *z_out, void *scratch, void *stream);
+
+/* ---- part 2: plane / line feature gather ---------------------------------------------
+ * Explicit normalised coordinates (isolated gather):
+ *   lm_gather_density_xyz  out[M]        = sum_k sum_c plane_k,c(x) * line_k,c(x)
+ *                          GridNeRF.compute_densityfeature, gridnerf_sequential.py:779-827;
+ *                          prior art compute_appfeature.gridsample_sum_xyz_b
+ *   lm_gather_app_xyz      out[M, n*C]   = plane_k,c(x) * line_k,c(x), column k*C + c
+ *                          GridNeRF.compute_appfeature before basis_mat,
+ *                          gridnerf_sequential.py:829-864; prior art gridsample_ew_xyb_bz
+ */
+int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
+                          void *stream);
+int lm_gather_app_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
+                      void *stream);
+
+/* ---- part 3: colour network ----------------------------------------------------------
+ * MLPRender_Fea.forward (app/models/mlp_render_fea.py:44-68) with positional_encoding
+ * (app/tools/utils.py:42-48): rgb = sigmoid(L3(relu(L2(relu(L1([feat|view|PE(feat)|PE(view)])))))).
+ * Supported shape: app_dim 27, view_pe = fea_pe = 2 (input 150), hidden 128, encode_app off.
+ * lm_mlp_pack (HOST memory in and out) reorders basis_mat [27,K] and the three Linear
+ * layers into the matrix-core fragment order the kernels read; biases may be NULL.
+ * prior art: pe_concate + gemm_fp16.run x3 (dist_render/kernel/cuda_render_extend.py:461-498).
+ */
+size_t lm_mlp_packed_bytes(int32_t prec, int32_t K_basis);
+int lm_mlp_pack(int32_t prec, int32_t K_basis, const float *basis, const float *w1, const float *b1,
+                const float *w2, const float *b2, const float *w3, const float *b3, void *packed_out);
+/* feat [M,27] fp32, view [M,3] fp32 -> rgb [M,3] fp32 */
+int lm_mlp(int32_t prec, const void *packed, int32_t K_basis, const float *feat, const float *view, int64_t M,
+           float *rgb, void *stream);
+/* products [M,K] fp32 -> feat [M,27] fp32 : basis_mat(products), gridnerf_sequential.py:871 */
+int lm_basis(int32_t prec, const void *packed, int32_t K_basis, const float *products, int64_t M, float *feat,
+             void *stream);
+
+/* ---- part 4: compositing -------------------------------------------------------------
+ * raw2alpha (app/tools/utils.py:51-64) on sigma scattered by the valid list, the weight
+ * threshold (gridnerf_sequential.py:479/553) and the sums of :493-504 / :565-576;
+ * prior art compute_beta.cuda + compute_weight.cuda (dist_render/kernel/cuda_kernel/volrend).
+ *   sigma       [n_valid] densities of the valid samples, in valid-list order
+ *   weight_out  optional [N*S] dense weights (NULL to skip)
+ *   app_bits    [N * ceil(S/64)] uint64: bit l of word (r, c) = sample 64c+l of ray r has weight > thres
+ *   app_base    [N * ceil(S/64)] uint32: slot of the first such sample of that word in app_idx
+ *   app_idx     [capacity N*S] uint32 flat indices of those samples (slot order)
+ *   app_w       [capacity N*S] float their weights
+ *   acc, depth  [N]
+ */
+int lm_weights(const lm_geom *geom, const float *rays, int64_t N, const uint64_t *bitmap,
+               const uint32_t *word_prefix, const float *sigma, float distance_scale, float weight_thres,
+               float term_eps, float *weight_out, uint64_t *app_bits, uint32_t *app_base, uint32_t *app_idx,
+               float *app_w, float *acc, float *depth, uint32_t *counters, void *stream);
+
+/* ---- whole chunk ---------------------------------------------------------------------
+ * GridBaseSequential.forward(rays_chunk, white_bg, is_train=False)
+ * (gridnerf_sequential.py:439-658) -> rgb_map [N,3], depth_map [N].
+ * workspace: lm_render_workspace_bytes(N, S, K_app) bytes of device memory, reusable
+ * across calls (the role of MultiBlockParallelCuda.allocate_tensors,
+ * dist_render/kernel/cuda_render_extend.py:35-159).  counters: [LM_STAT_WORDS] uint32
+ * device memory, may be NULL.  No host synchronisation happens inside. */
+size_t lm_render_workspace_bytes(int64_t N, int32_t S, int32_t K_app);
+int lm_render(const lm_model *model, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
+              float *rgb_map, float *depth_map, uint32_t *counters, void *stream);
+
+/* Stage-level pieces of lm_render for validation and profiling (same kernels). */
+int lm_density_valid(const lm_model *model, const float *rays, const uint32_t *valid_idx,
+                     const uint32_t *counters, float *sigma, void *stream);
+int lm_app_products(const lm_model *model, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
+                    float *products, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LANDMARK_HIP_H */

@@ -1,0 +1,167 @@
+// C-ABI plumbing: error string, launch sizing, table relayout and the whole-chunk render.
+#include <stdarg.h>
+
+#include <algorithm>
+
+#include "lm_common.h"
+
+static thread_local char g_err[512] = "";
+
+void lm_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char *lm_last_error(void) { return g_err; }
+extern "C" int lm_abi_version(void) { return LM_ABI_VERSION; }
+
+int lm_persistent_blocks(int blocks_per_cu) {
+    static thread_local int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus * blocks_per_cu;
+}
+
+// ---- [C,H,W] -> [H,W,C] ---------------------------------------------------------------------
+namespace {
+template <typename T>
+__global__ __launch_bounds__(256) void k_relayout(const T *__restrict__ src, T *__restrict__ dst, int C, uint64_t HW) {
+    // 64 texels x 64 channels per tile through LDS: coalesced reads along HW, coalesced writes along C
+    __shared__ T tile[64][65];
+    const uint64_t t0 = (uint64_t)blockIdx.x * 64;
+    const int c0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int cc = ty; cc < 64; cc += 4) {
+        const int c = c0 + cc;
+        const uint64_t t = t0 + tx;
+        if (c < C && t < HW) tile[cc][tx] = src[(uint64_t)c * HW + t];
+    }
+    __syncthreads();
+    for (int tt = ty; tt < 64; tt += 4) {
+        const uint64_t t = t0 + tt;
+        const int c = c0 + tx;
+        if (c < C && t < HW) dst[t * C + c] = tile[tx][tt];
+    }
+}
+}  // namespace
+
+extern "C" int lm_relayout_nchw_to_hwc(const void *src, void *dst, int32_t C, int32_t H, int32_t W, int32_t dtype,
+                                       void *stream) {
+    LM_REQUIRE(src && dst && src != dst, "null or aliased buffer");
+    LM_REQUIRE(C > 0 && H > 0 && W > 0, "empty table");
+    LM_REQUIRE(dtype == LM_F32 || dtype == LM_F16, "unknown dtype %d", dtype);
+    const uint64_t HW = (uint64_t)H * (uint64_t)W;
+    const uint64_t bx = (HW + 63) / 64;
+    LM_REQUIRE(bx < (1ull << 31), "table too large");
+    dim3 grid((unsigned)bx, (unsigned)((C + 63) / 64));
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_relayout<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float *)src, (float *)dst, C, HW);
+    else
+        hipLaunchKernelGGL(k_relayout<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)src,
+                           (uint16_t *)dst, C, HW);
+    LM_CHECK_LAUNCH("k_relayout");
+    return LM_OK;
+}
+
+// ---- whole chunk -------------------------------------------------------------------------------
+int lm_check_geom(const lm_geom *g);
+int lm_check_planes(const lm_plane *planes, int32_t n, int *dtype_out, int *K_out);
+int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *products, const float *rays,
+                         const uint32_t *app_idx, const uint32_t *count, float *rgb, hipStream_t stream);
+int lm_launch_composite(int64_t N, int S, const uint64_t *app_bits, const uint32_t *app_base, const float *app_w,
+                        const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream);
+int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
+
+namespace {
+struct Workspace {
+    uint64_t *bitmap;
+    uint32_t *word_prefix;
+    void *cull_scratch;
+    uint32_t *valid_idx;
+    float *sigma;
+    uint64_t *app_bits;
+    uint32_t *app_base;
+    uint32_t *app_idx;
+    float *app_w;
+    float *rgb;
+    float *products;
+    float *acc;
+    uint32_t *counters;
+    size_t total;
+};
+
+Workspace carve(char *base, int64_t N, int32_t S, int32_t K) {
+    Workspace w;
+    size_t o = 0;
+    auto take = [&](size_t bytes) {
+        char *p = base ? base + o : nullptr;
+        o = (o + bytes + 255) & ~(size_t)255;
+        return p;
+    };
+    const uint64_t total = (uint64_t)N * (uint64_t)S, n_words = (total + 63) / 64, steps = (uint64_t)(S + 63) / 64;
+    // a ray's weights sum to at most 1, so at most min(S, 1/threshold) of them can exceed the
+    // threshold; without knowing the threshold the capacity is N*S
+    const uint64_t cap = total;
+    w.bitmap = (uint64_t *)take(n_words * 8);
+    w.word_prefix = (uint32_t *)take(n_words * 4);
+    w.cull_scratch = take(lm_sample_cull_scratch_bytes(N, S));
+    w.valid_idx = (uint32_t *)take(total * 4);
+    w.sigma = (float *)take(total * 4);
+    w.app_bits = (uint64_t *)take((uint64_t)N * steps * 8);
+    w.app_base = (uint32_t *)take((uint64_t)N * steps * 4);
+    w.app_idx = (uint32_t *)take(cap * 4);
+    w.app_w = (float *)take(cap * 4);
+    w.rgb = (float *)take(cap * 12);
+    w.products = (float *)take(cap * (uint64_t)K * 4);
+    w.acc = (float *)take((uint64_t)N * 4);
+    w.counters = (uint32_t *)take(LM_STAT_WORDS * 4);
+    w.total = o;
+    return w;
+}
+}  // namespace
+
+extern "C" size_t lm_render_workspace_bytes(int64_t N, int32_t S, int32_t K_app) {
+    if (N <= 0 || S <= 0 || K_app <= 0) return 0;
+    return carve(nullptr, N, S, K_app).total;
+}
+
+extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
+                         float *rgb_map, float *depth_map, uint32_t *counters, void *stream) {
+    LM_REQUIRE(m != nullptr, "model is null");
+    if (int rc = lm_check_geom(&m->geom)) return rc;
+    int dt, K;
+    if (int rc = lm_check_planes(m->density, m->n_planes, &dt, nullptr)) return rc;
+    if (int rc = lm_check_planes(m->app, m->n_planes, &dt, &K)) return rc;
+    LM_REQUIRE(N >= 0, "negative ray count");
+    if (N == 0) return LM_OK;
+    LM_REQUIRE(rays && rgb_map && depth_map, "null buffer");
+    LM_REQUIRE(workspace && lm_aligned16(workspace), "workspace is null or misaligned");
+    const int S = m->geom.S;
+    LM_REQUIRE((uint64_t)N * (uint64_t)S < (1ull << 32), "N*S does not fit 32-bit sample indices; split the chunk");
+    Workspace w = carve((char *)workspace, N, S, K);
+    if (w.total > workspace_bytes)
+        LM_FAIL(LM_ERR_WORKSPACE, "workspace has %zu bytes, %zu needed for N=%lld S=%d K=%d", workspace_bytes, w.total,
+                (long long)N, S, K);
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *cnt = counters ? counters : w.counters;
+    if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
+    if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, w.valid_idx, cnt, nullptr, w.cull_scratch, st))
+        return rc;
+    if (int rc = lm_density_valid(m, rays, w.valid_idx, cnt, w.sigma, st)) return rc;
+    if (int rc = lm_weights(&m->geom, rays, N, w.bitmap, w.word_prefix, w.sigma, m->distance_scale, m->weight_thres,
+                            m->term_eps, nullptr, w.app_bits, w.app_base, w.app_idx, w.app_w, w.acc, depth_map, cnt, st))
+        return rc;
+    if (int rc = lm_app_products(m, rays, w.app_idx, cnt, w.products, st)) return rc;
+    if (int rc = lm_launch_app_colour(m->mlp_prec, m->mlp_packed, K, S, w.products, rays, w.app_idx,
+                                      cnt + LM_STAT_N_APP, w.rgb, st))
+        return rc;
+    return lm_launch_composite(N, S, w.app_bits, w.app_base, w.app_w, w.rgb, w.acc, m->white_bg, rgb_map, st);
+}

@@ -1,0 +1,154 @@
+// Shared declarations of the gfx950 kernels behind include/landmark_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/landmark_hip.h"
+
+#define LM_WAVE 64
+
+// Error plumbing: thread-local message, negative status.
+void lm_set_error(const char *fmt, ...);
+#define LM_FAIL(code, ...)         \
+    do {                           \
+        lm_set_error(__VA_ARGS__); \
+        return (code);             \
+    } while (0)
+#define LM_REQUIRE(cond, ...)                               \
+    do {                                                    \
+        if (!(cond)) LM_FAIL(LM_ERR_INVALID, __VA_ARGS__);  \
+    } while (0)
+#define LM_CHECK_LAUNCH(name)                                                              \
+    do {                                                                                   \
+        hipError_t e_ = hipGetLastError();                                                 \
+        if (e_ != hipSuccess) LM_FAIL(LM_ERR_LAUNCH, "%s: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+static inline bool lm_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Number of workgroups for grid-stride kernels: enough resident waves to cover every CU
+// several times over; 256 CUs in 8 XCDs on MI355X.
+int lm_persistent_blocks(int blocks_per_cu);
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Remap the
+// hardware block id so that blocks resident on one XCD own neighbouring tiles.
+__device__ __forceinline__ unsigned lm_xcd_swizzle(unsigned bid, unsigned nblocks) {
+    const unsigned nx = 8;
+    if (nblocks % nx) return bid;
+    return (bid % nx) * (nblocks / nx) + bid / nx;
+}
+
+// ---------------------------------------------------------------------------------------
+// Geometry with the reference's rounding: every product and sum is a separate float
+// operation (the translation unit is built with -ffp-contract=off), divisions are IEEE.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float lm_ray_param(const lm_geom &g, const float *ray) {
+    if (g.sampler == LM_SAMPLER_HULL) {
+        float o_z = ray[2] - g.aabb[2];
+        float far = -(o_z / ray[5]);
+        if (ray[5] >= 0.0f) far = g.far_;
+        return far;
+    }
+    float tmin = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        float v = ray[3 + k] == 0.0f ? 1e-6f : ray[3 + k];
+        float ra = (g.aabb[3 + k] - ray[k]) / v;
+        float rb = (g.aabb[k] - ray[k]) / v;
+        float m = ra < rb ? ra : rb;
+        if (ra != ra || rb != rb) m = NAN;
+        if (m > tmin || m != m) tmin = m;
+    }
+    if (tmin < g.near_) tmin = g.near_;
+    if (tmin > g.far_) tmin = g.far_;
+    return tmin;
+}
+
+__device__ __forceinline__ float lm_sample_z(const lm_geom &g, float ray_param, int s) {
+    if (g.sampler == LM_SAMPLER_HULL) {
+        float b = ray_param * g.tab_t[s];
+        return g.tab_a[s] + b;
+    }
+    return ray_param + g.tab_a[s];
+}
+
+__device__ __forceinline__ void lm_point(const float *ray, float z, float *pt) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        float m = ray[3 + k] * z;
+        pt[k] = ray[k] + m;
+    }
+}
+
+__device__ __forceinline__ bool lm_inside(const lm_geom &g, const float *pt) {
+    bool out = false;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) out |= (g.aabb[k] > pt[k]) | (pt[k] > g.aabb[3 + k]);
+    return !out;
+}
+
+__device__ __forceinline__ void lm_normalise(const lm_geom &g, const float *pt, float *q) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        float d = pt[k] - g.aabb[k];
+        float m = d * g.inv_aabb[k];
+        q[k] = m - 1.0f;
+    }
+}
+
+// Trilinear lookup with zero padding and align_corners=True in ATen's operation order
+// (corner order tnw, tne, tsw, tse, bnw, bne, bsw, bse; weight = (x)(y)(z) left to right;
+// each value*weight rounded before it is added).
+__device__ __forceinline__ float lm_alpha_lookup(const lm_geom &g, const float *pt) {
+    float c[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        float d = pt[k] - g.vol_aabb_min[k];
+        float m = d * g.vol_inv[k];
+        c[k] = m - 1.0f;
+    }
+    const int W = g.vw, H = g.vh, D = g.vd;
+    float ix = ((c[0] + 1.0f) / 2.0f) * (float)(W - 1);
+    float iy = ((c[1] + 1.0f) / 2.0f) * (float)(H - 1);
+    float iz = ((c[2] + 1.0f) / 2.0f) * (float)(D - 1);
+    float fx = floorf(ix), fy = floorf(iy), fz = floorf(iz);
+    float wx[2] = {(fx + 1.0f) - ix, ix - fx};
+    float wy[2] = {(fy + 1.0f) - iy, iy - fy};
+    float wz[2] = {(fz + 1.0f) - iz, iz - fz};
+    // clamp before the int conversion so that far-away points cannot overflow
+    fx = fminf(fmaxf(fx, -2.0f), (float)W);
+    fy = fminf(fmaxf(fy, -2.0f), (float)H);
+    fz = fminf(fmaxf(fz, -2.0f), (float)D);
+    int x0 = (int)fx, y0 = (int)fy, z0 = (int)fz;
+    float out = 0.0f;
+#pragma unroll
+    for (int zz = 0; zz < 2; ++zz)
+#pragma unroll
+        for (int yy = 0; yy < 2; ++yy)
+#pragma unroll
+            for (int xx = 0; xx < 2; ++xx) {
+                int x = x0 + xx, y = y0 + yy, z = z0 + zz;
+                if (x >= 0 && x < W && y >= 0 && y < H && z >= 0 && z < D) {
+                    float w = (wx[xx] * wy[yy]) * wz[zz];
+                    float t = g.vol[((size_t)z * H + y) * W + x] * w;
+                    out = out + t;
+                }
+            }
+    return out;
+}
+
+// Sample validity = inside the AABB and (no volume or lookup > threshold)
+__device__ __forceinline__ bool lm_sample_valid(const lm_geom &g, const float *pt) {
+    bool ok = lm_inside(g, pt);
+    if (ok && g.vol) ok = lm_alpha_lookup(g, pt) > g.vol_thre;
+    return ok;
+}
+
+// ---------------------------------------------------------------------------------------
+// wave64 helpers
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned lm_lane() { return __lane_id(); }
+__device__ __forceinline__ unsigned lm_mbcnt(uint64_t mask) {  // set bits of mask below this lane
+    return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
+}

@@ -1,0 +1,351 @@
+// Part 2: bilinear plane x linear line feature gather over channel-last tables.
+//
+// Four lanes share one sample.  Lane q of the quad owns channels [V*q, V*q+V) of every
+// group of 4V channels (V = 4 floats or 8 halves = one 16-byte load), so the quad reads
+// 64 contiguous bytes per load instruction and a corner of a 16-channel fp32 plane is one
+// such read.  All planes of all resolution levels are walked inside one launch; the
+// per-plane partial sums stay in registers.  Work is a grid-stride loop over tiles of 64
+// samples so the launch shape does not depend on counts that only exist on the device.
+//
+// Interpolation follows F.grid_sample(align_corners=True, zeros padding) as the reference
+// calls it (app/models/gridnerf_sequential.py:803-812, 851-862): unnormalise
+// ((c+1)/2)*(size-1), corners floor/floor+1, out-of-range corners contribute zero.
+#include <hip/hip_fp16.h>
+
+#include "lm_common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kQuad = 4;
+constexpr int kTile = kBlock / kQuad;  // samples per workgroup iteration
+
+struct PlaneSet {
+    lm_plane p[LM_MAX_PLANES];
+    int n;
+};
+
+template <typename T> struct Vec;
+template <> struct Vec<float> {
+    static constexpr int V = 4;
+    __device__ static __forceinline__ void load(const float *p, float *o) {
+        float4 v = *reinterpret_cast<const float4 *>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct Vec<__half> {
+    static constexpr int V = 8;
+    __device__ static __forceinline__ void load(const __half *p, float *o) {
+        uint4 raw = *reinterpret_cast<const uint4 *>(p);
+        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float2 f = __half22float2(h[i]);
+            o[2 * i] = f.x; o[2 * i + 1] = f.y;
+        }
+    }
+};
+
+struct Taps2 {  // bilinear footprint: element offsets of the 4 corners and their weights
+    int64_t o00, o01, o10, o11;
+    float w00, w01, w10, w11;
+};
+struct Taps1 {
+    int o0, o1;
+    float w0, w1;
+};
+
+__device__ __forceinline__ float unnorm(float c, int size) { return ((c + 1.0f) / 2.0f) * (float)(size - 1); }
+
+__device__ __forceinline__ Taps2 plane_taps(const lm_plane &pl, float cx, float cy) {
+    const float ix = unnorm(cx, pl.W), iy = unnorm(cy, pl.H);
+    const float fx = floorf(ix), fy = floorf(iy);
+    float wx1 = ix - fx, wx0 = (fx + 1.0f) - ix, wy1 = iy - fy, wy0 = (fy + 1.0f) - iy;
+    // clamp in float first: coordinates far outside the table must not overflow the int cast
+    int x0 = (int)fminf(fmaxf(fx, -2.0f), (float)pl.W), y0 = (int)fminf(fmaxf(fy, -2.0f), (float)pl.H);
+    int x1 = x0 + 1, y1 = y0 + 1;
+    if (x0 < 0 || x0 >= pl.W) wx0 = 0.0f;
+    if (x1 < 0 || x1 >= pl.W) wx1 = 0.0f;
+    if (y0 < 0 || y0 >= pl.H) wy0 = 0.0f;
+    if (y1 < 0 || y1 >= pl.H) wy1 = 0.0f;
+    x0 = min(max(x0, 0), pl.W - 1); x1 = min(max(x1, 0), pl.W - 1);
+    y0 = min(max(y0, 0), pl.H - 1); y1 = min(max(y1, 0), pl.H - 1);
+    Taps2 t;
+    const int64_t r0 = (int64_t)y0 * pl.W, r1 = (int64_t)y1 * pl.W;
+    t.o00 = (r0 + x0) * pl.C; t.o01 = (r0 + x1) * pl.C;
+    t.o10 = (r1 + x0) * pl.C; t.o11 = (r1 + x1) * pl.C;
+    t.w00 = wx0 * wy0; t.w01 = wx1 * wy0; t.w10 = wx0 * wy1; t.w11 = wx1 * wy1;
+    return t;
+}
+
+__device__ __forceinline__ Taps1 line_taps(const lm_plane &pl, float c) {
+    const float i = unnorm(c, pl.Len);
+    const float f = floorf(i);
+    float w1 = i - f, w0 = (f + 1.0f) - i;
+    int i0 = (int)fminf(fmaxf(f, -2.0f), (float)pl.Len), i1 = i0 + 1;
+    if (i0 < 0 || i0 >= pl.Len) w0 = 0.0f;
+    if (i1 < 0 || i1 >= pl.Len) w1 = 0.0f;
+    i0 = min(max(i0, 0), pl.Len - 1); i1 = min(max(i1, 0), pl.Len - 1);
+    Taps1 t;
+    t.o0 = i0 * pl.C; t.o1 = i1 * pl.C;
+    t.w0 = w0; t.w1 = w1;
+    return t;
+}
+
+__device__ __forceinline__ float pick(const float *q, int ax) { return ax == 0 ? q[0] : (ax == 1 ? q[1] : q[2]); }
+
+// products of one plane for the V channels starting at c (lane-private)
+template <typename T>
+__device__ __forceinline__ void plane_products(const lm_plane &pl, const Taps2 &t2, const Taps1 &t1, int c, float *prod) {
+    constexpr int V = Vec<T>::V;
+    const T *P = reinterpret_cast<const T *>(pl.plane);
+    const T *Ln = reinterpret_cast<const T *>(pl.line);
+    float a[V], b[V], cc[V], d[V], l0[V], l1[V];
+    Vec<T>::load(P + t2.o00 + c, a);
+    Vec<T>::load(P + t2.o01 + c, b);
+    Vec<T>::load(P + t2.o10 + c, cc);
+    Vec<T>::load(P + t2.o11 + c, d);
+    Vec<T>::load(Ln + t1.o0 + c, l0);
+    Vec<T>::load(Ln + t1.o1 + c, l1);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+        float pv = a[i] * t2.w00;
+        pv = fmaf(b[i], t2.w01, pv);
+        pv = fmaf(cc[i], t2.w10, pv);
+        pv = fmaf(d[i], t2.w11, pv);
+        float lv = fmaf(l1[i], t1.w1, l0[i] * t1.w0);
+        prod[i] = pv * lv;
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q, unsigned qlane) {
+    constexpr int V = Vec<T>::V;
+    float sum = 0.0f;
+    for (int k = 0; k < ps.n; ++k) {
+        const lm_plane &pl = ps.p[k];
+        const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+        const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        for (int c = V * qlane; c < pl.C; c += V * kQuad) {
+            float prod[V];
+            plane_products<T>(pl, t2, t1, c, prod);
+#pragma unroll
+            for (int i = 0; i < V; ++i) sum += prod[i];
+        }
+    }
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    return sum;
+}
+
+template <typename T>
+__device__ __forceinline__ void app_store(const PlaneSet &ps, const float *q, unsigned qlane, float *row) {
+    constexpr int V = Vec<T>::V;
+    int col = 0;
+    for (int k = 0; k < ps.n; ++k) {
+        const lm_plane &pl = ps.p[k];
+        const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+        const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        for (int c = V * qlane; c < pl.C; c += V * kQuad) {
+            float prod[V];
+            plane_products<T>(pl, t2, t1, c, prod);
+#pragma unroll
+            for (int i = 0; i < V; i += 4)
+                *reinterpret_cast<float4 *>(row + col + c + i) = make_float4(prod[i], prod[i + 1], prod[i + 2], prod[i + 3]);
+        }
+        col += pl.C;
+    }
+}
+
+// coordinates of list entry `flat` (= ray*S + s): same operations as the sampler
+__device__ __forceinline__ void list_coords(const lm_geom &g, const float *__restrict__ rays, uint32_t flat, float *q) {
+    const uint32_t r = flat / (uint32_t)g.S;
+    const int s = (int)(flat - r * (uint32_t)g.S);
+    float ray[6];
+    const float2 *rp = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
+    float2 a = rp[0], b = rp[1], c = rp[2];
+    ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+    const float z = lm_sample_z(g, lm_ray_param(g, ray), s);
+    float pt[3];
+    lm_point(ray, z, pt);
+    lm_normalise(g, pt, q);
+}
+
+__device__ __forceinline__ float activate(float f, int act, float shift) {
+    if (act == LM_ACT_SOFTPLUS) {
+        const float x = f + shift;
+        return x > 20.0f ? x : log1pf(expf(x));
+    }
+    return fmaxf(f, 0.0f);
+}
+
+// ---- explicit coordinates ----------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float *__restrict__ xyz, uint64_t M,
+                                                        float *__restrict__ out) {
+    const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
+    const uint64_t n_tiles = (M + kTile - 1) / kTile;
+    for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
+        const uint64_t p = tile * kTile + slot;
+        if (p >= M) continue;
+        float q[3] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2]};
+        const float s = density_sum<T>(ps, q, qlane);
+        if (qlane == 0) out[p] = s;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_app_xyz(PlaneSet ps, int K, const float *__restrict__ xyz, uint64_t M,
+                                                    float *__restrict__ out) {
+    const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
+    const uint64_t n_tiles = (M + kTile - 1) / kTile;
+    for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
+        const uint64_t p = tile * kTile + slot;
+        if (p >= M) continue;
+        float q[3] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2]};
+        app_store<T>(ps, q, qlane, out + p * (uint64_t)K);
+    }
+}
+
+// ---- list driven (inside the render) -------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps, const float *__restrict__ rays,
+                                                         const uint32_t *__restrict__ list,
+                                                         const uint32_t *__restrict__ count, int act, float shift,
+                                                         float *__restrict__ sigma) {
+    const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
+    const uint64_t M = *count;
+    const uint64_t n_tiles = (M + kTile - 1) / kTile;
+    for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
+        const uint64_t p = tile * kTile + slot;
+        if (p >= M) continue;
+        float q[3];
+        list_coords(g, rays, list[p], q);
+        const float s = density_sum<T>(ps, q, qlane);
+        if (qlane == 0) sigma[p] = activate(s, act, shift);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int K, const float *__restrict__ rays,
+                                                     const uint32_t *__restrict__ list,
+                                                     const uint32_t *__restrict__ count, float *__restrict__ out) {
+    const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
+    const uint64_t M = *count;
+    const uint64_t n_tiles = (M + kTile - 1) / kTile;
+    for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
+        const uint64_t p = tile * kTile + slot;
+        if (p >= M) continue;
+        float q[3];
+        list_coords(g, rays, list[p], q);
+        app_store<T>(ps, q, qlane, out + p * (uint64_t)K);
+    }
+}
+
+}  // namespace
+
+// -------------------------------------------------------------------------------------------
+int lm_check_planes(const lm_plane *planes, int32_t n, int *dtype_out, int *K_out) {
+    LM_REQUIRE(planes != nullptr, "planes is null");
+    LM_REQUIRE(n >= 1 && n <= LM_MAX_PLANES, "n_planes %d out of range 1..%d", n, LM_MAX_PLANES);
+    int K = 0;
+    for (int k = 0; k < n; ++k) {
+        const lm_plane &p = planes[k];
+        LM_REQUIRE(p.plane && p.line, "plane %d: null table", k);
+        LM_REQUIRE(lm_aligned16(p.plane) && lm_aligned16(p.line), "plane %d: tables must be 16-byte aligned", k);
+        LM_REQUIRE(p.H > 0 && p.W > 0 && p.Len > 0, "plane %d: empty table", k);
+        LM_REQUIRE(p.dtype == planes[0].dtype, "planes must share one storage type");
+        LM_REQUIRE(p.dtype == LM_F32 || p.dtype == LM_F16, "plane %d: unknown dtype %d", k, p.dtype);
+        const int V = p.dtype == LM_F32 ? 4 : 8;
+        LM_REQUIRE(p.C > 0 && p.C % V == 0, "plane %d: channel count %d must be a multiple of %d", k, p.C, V);
+        LM_REQUIRE(p.ax0 >= 0 && p.ax0 < 3 && p.ax1 >= 0 && p.ax1 < 3 && p.axl >= 0 && p.axl < 3, "plane %d: bad axis", k);
+        K += p.C;
+    }
+    *dtype_out = planes[0].dtype;
+    if (K_out) *K_out = K;
+    return LM_OK;
+}
+
+static PlaneSet make_set(const lm_plane *planes, int n) {
+    PlaneSet ps;
+    for (int k = 0; k < LM_MAX_PLANES; ++k) ps.p[k] = planes[k < n ? k : 0];
+    ps.n = n;
+    return ps;
+}
+
+extern "C" int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
+                                     void *stream) {
+    int dtype;
+    if (int rc = lm_check_planes(planes, n_planes, &dtype, nullptr)) return rc;
+    LM_REQUIRE(M >= 0, "negative count");
+    if (M == 0) return LM_OK;
+    LM_REQUIRE(xyz && out, "null buffer");
+    const PlaneSet ps = make_set(planes, n_planes);
+    const uint64_t tiles = ((uint64_t)M + kTile - 1) / kTile;
+    const unsigned grid = (unsigned)std::min<uint64_t>(tiles, (uint64_t)lm_persistent_blocks(8));
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_density_xyz<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, xyz, (uint64_t)M, out);
+    else
+        hipLaunchKernelGGL(k_density_xyz<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, xyz, (uint64_t)M, out);
+    LM_CHECK_LAUNCH("k_density_xyz");
+    return LM_OK;
+}
+
+extern "C" int lm_gather_app_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
+                                 void *stream) {
+    int dtype, K;
+    if (int rc = lm_check_planes(planes, n_planes, &dtype, &K)) return rc;
+    LM_REQUIRE(M >= 0, "negative count");
+    if (M == 0) return LM_OK;
+    LM_REQUIRE(xyz && out && lm_aligned16(out), "null or misaligned buffer");
+    const PlaneSet ps = make_set(planes, n_planes);
+    const uint64_t tiles = ((uint64_t)M + kTile - 1) / kTile;
+    const unsigned grid = (unsigned)std::min<uint64_t>(tiles, (uint64_t)lm_persistent_blocks(8));
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_app_xyz<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, K, xyz, (uint64_t)M, out);
+    else
+        hipLaunchKernelGGL(k_app_xyz<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, K, xyz, (uint64_t)M, out);
+    LM_CHECK_LAUNCH("k_app_xyz");
+    return LM_OK;
+}
+
+int lm_check_geom(const lm_geom *g);
+
+extern "C" int lm_density_valid(const lm_model *m, const float *rays, const uint32_t *valid_idx,
+                                const uint32_t *counters, float *sigma, void *stream) {
+    LM_REQUIRE(m != nullptr, "model is null");
+    if (int rc = lm_check_geom(&m->geom)) return rc;
+    int dtype;
+    if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
+    LM_REQUIRE(rays && valid_idx && counters && sigma, "null buffer");
+    LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
+    const PlaneSet ps = make_set(m->density, m->n_planes);
+    const unsigned grid = (unsigned)lm_persistent_blocks(8);
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_density_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, rays,
+                           valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
+    else
+        hipLaunchKernelGGL(k_density_list<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, rays,
+                           valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
+    LM_CHECK_LAUNCH("k_density_list");
+    return LM_OK;
+}
+
+extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
+                               float *products, void *stream) {
+    LM_REQUIRE(m != nullptr, "model is null");
+    if (int rc = lm_check_geom(&m->geom)) return rc;
+    int dtype, K;
+    if (int rc = lm_check_planes(m->app, m->n_planes, &dtype, &K)) return rc;
+    LM_REQUIRE(rays && app_idx && counters && products && lm_aligned16(products), "null or misaligned buffer");
+    const PlaneSet ps = make_set(m->app, m->n_planes);
+    const unsigned grid = (unsigned)lm_persistent_blocks(8);
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_app_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, K, rays,
+                           app_idx, counters + LM_STAT_N_APP, products);
+    else
+        hipLaunchKernelGGL(k_app_list<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, K, rays,
+                           app_idx, counters + LM_STAT_N_APP, products);
+    LM_CHECK_LAUNCH("k_app_list");
+    return LM_OK;
+}

@@ -1,0 +1,168 @@
+// Part 1: ray sampling, AABB / occupancy culling and stable compaction.
+//
+// Samples are numbered ray*S + s.  A wave owns 64 consecutive samples, decides their
+// validity, and stores the 64 decisions as one bitmap word (wave ballot).  Compaction is
+// a prefix sum over the words' popcounts:
+//   k_sample_cull  bitmap words + one popcount per workgroup (4096 samples)
+//   k_scan_blocks  exclusive scan of the workgroup counts (one workgroup), total -> counters
+//   k_emit         per-word prefix and the ascending list of valid flat indices
+// The list order is the row-major order of the reference's boolean-mask indexing
+// (app/models/gridnerf_sequential.py:461-465, 472), so indices match it exactly.
+#include "lm_common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWordsPerBlock = 64;  // 4096 samples per workgroup
+constexpr int kWordsPerWave = kWordsPerBlock / (kBlock / LM_WAVE);
+
+__global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *__restrict__ rays, uint64_t total,
+                                                        uint64_t n_words, uint64_t *__restrict__ bitmap,
+                                                        uint32_t *__restrict__ block_count, float *__restrict__ z_out) {
+    __shared__ uint32_t s_cnt[kBlock / LM_WAVE];
+    const unsigned lane = lm_lane();
+    const unsigned wave = threadIdx.x / LM_WAVE;
+    const uint64_t w0 = (uint64_t)blockIdx.x * kWordsPerBlock + (uint64_t)wave * kWordsPerWave;
+    uint32_t cnt = 0;
+    for (int it = 0; it < kWordsPerWave; ++it) {
+        const uint64_t w = w0 + it;
+        if (w >= n_words) break;
+        const uint64_t flat = w * 64 + lane;
+        bool ok = false;
+        if (flat < total) {
+            const uint64_t r = flat / (uint32_t)g.S;
+            const int s = (int)(flat - r * (uint32_t)g.S);
+            float ray[6];
+            const float2 *rp = reinterpret_cast<const float2 *>(rays + 6 * r);
+            float2 a = rp[0], b = rp[1], c = rp[2];
+            ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+            const float z = lm_sample_z(g, lm_ray_param(g, ray), s);
+            float pt[3];
+            lm_point(ray, z, pt);
+            ok = lm_sample_valid(g, pt);
+            if (z_out) z_out[flat] = z;
+        }
+        const uint64_t bits = __ballot(ok);
+        if (lane == 0) bitmap[w] = bits;
+        cnt += (uint32_t)__popcll(bits);
+    }
+    if (lane == 0) s_cnt[wave] = cnt;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t t = 0;
+        for (int i = 0; i < kBlock / LM_WAVE; ++i) t += s_cnt[i];
+        block_count[blockIdx.x] = t;
+    }
+}
+
+// exclusive scan of n counts by one workgroup of 1024 threads; total -> *total_out
+__global__ __launch_bounds__(1024) void k_scan_blocks(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
+                                                      uint32_t n, uint32_t *__restrict__ total_out) {
+    __shared__ uint32_t s_wave[16];
+    __shared__ uint32_t s_carry;
+    const unsigned lane = lm_lane(), wave = threadIdx.x / LM_WAVE;
+    if (threadIdx.x == 0) s_carry = 0;
+    __syncthreads();
+    for (uint32_t base = 0; base < n; base += 1024) {
+        const uint32_t i = base + threadIdx.x;
+        const uint32_t v = i < n ? in[i] : 0;
+        uint32_t x = v;  // inclusive wave scan
+#pragma unroll
+        for (int d = 1; d < LM_WAVE; d <<= 1) {
+            uint32_t y = __shfl_up(x, d);
+            if (lane >= (unsigned)d) x += y;
+        }
+        if (lane == LM_WAVE - 1) s_wave[wave] = x;
+        __syncthreads();
+        uint32_t off = s_carry;
+        for (unsigned k = 0; k < wave; ++k) off += s_wave[k];
+        if (i < n) out[i] = off + x - v;
+        __syncthreads();
+        if (threadIdx.x == 1023) s_carry = off + x;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *total_out = s_carry;
+}
+
+__global__ __launch_bounds__(kBlock) void k_emit(const uint64_t *__restrict__ bitmap, uint64_t n_words,
+                                                 const uint32_t *__restrict__ block_off,
+                                                 uint32_t *__restrict__ word_prefix, uint32_t *__restrict__ valid_idx) {
+    __shared__ uint32_t s_pref[kWordsPerBlock];
+    const unsigned lane = lm_lane(), wave = threadIdx.x / LM_WAVE;
+    const uint64_t wb = (uint64_t)blockIdx.x * kWordsPerBlock;
+    if (wave == 0) {
+        const uint64_t w = wb + lane;
+        const uint32_t v = w < n_words ? (uint32_t)__popcll(bitmap[w]) : 0;
+        uint32_t x = v;
+#pragma unroll
+        for (int d = 1; d < LM_WAVE; d <<= 1) {
+            uint32_t y = __shfl_up(x, d);
+            if (lane >= (unsigned)d) x += y;
+        }
+        const uint32_t p = block_off[blockIdx.x] + x - v;
+        s_pref[lane] = p;
+        if (w < n_words) word_prefix[w] = p;
+    }
+    __syncthreads();
+    for (int it = 0; it < kWordsPerWave; ++it) {
+        const unsigned wi = wave * kWordsPerWave + it;
+        const uint64_t w = wb + wi;
+        if (w >= n_words) break;
+        const uint64_t bits = bitmap[w];
+        if ((bits >> lane) & 1ull) valid_idx[s_pref[wi] + lm_mbcnt(bits)] = (uint32_t)(w * 64 + lane);
+    }
+}
+
+}  // namespace
+
+static uint64_t n_blocks_for(uint64_t n_words) { return (n_words + kWordsPerBlock - 1) / kWordsPerBlock; }
+
+extern "C" size_t lm_sample_cull_scratch_bytes(int64_t N, int32_t S) {
+    if (N <= 0 || S <= 0) return 0;
+    const uint64_t n_words = ((uint64_t)N * (uint64_t)S + 63) / 64;
+    return (size_t)(n_blocks_for(n_words) * 2 * sizeof(uint32_t) + 256);
+}
+
+int lm_check_geom(const lm_geom *g) {
+    LM_REQUIRE(g != nullptr, "geom is null");
+    LM_REQUIRE(g->S > 0, "S must be positive (got %d)", g->S);
+    LM_REQUIRE(g->sampler == LM_SAMPLER_AABB || g->sampler == LM_SAMPLER_HULL, "unknown sampler %d", g->sampler);
+    LM_REQUIRE(g->tab_a && g->tab_t, "sampler tables are null");
+    if (g->vol) LM_REQUIRE(g->vd > 0 && g->vh > 0 && g->vw > 0, "occupancy volume has an empty dimension");
+    return LM_OK;
+}
+
+extern "C" int lm_sample_cull(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap,
+                              uint32_t *word_prefix, uint32_t *valid_idx, uint32_t *counters, float *z_out,
+                              void *scratch, void *stream) {
+    if (int rc = lm_check_geom(geom)) return rc;
+    LM_REQUIRE(N >= 0, "negative ray count");
+    LM_REQUIRE(counters != nullptr, "counters is null");
+    hipStream_t st = (hipStream_t)stream;
+    const uint64_t total = (uint64_t)N * (uint64_t)geom->S;
+    LM_REQUIRE(total < (1ull << 32), "N*S = %llu does not fit 32-bit sample indices; split the chunk",
+               (unsigned long long)total);
+    if (N == 0) {
+        // an empty chunk is valid (the reference's chunk loop never issues one, but a caller may)
+        hipLaunchKernelGGL(k_scan_blocks, dim3(1), dim3(1024), 0, st, (const uint32_t *)nullptr, (uint32_t *)nullptr, 0u,
+                           counters + LM_STAT_N_VALID);
+        LM_CHECK_LAUNCH("k_scan_blocks");
+        return LM_OK;
+    }
+    LM_REQUIRE(rays && bitmap && word_prefix && valid_idx && scratch, "null buffer");
+    LM_REQUIRE(lm_aligned16(rays) && lm_aligned16(bitmap) && lm_aligned16(scratch), "buffers must be 16-byte aligned");
+    const uint64_t n_words = (total + 63) / 64;
+    const uint64_t nb = n_blocks_for(n_words);
+    uint32_t *block_count = (uint32_t *)scratch;
+    uint32_t *block_off = block_count + nb;
+    hipLaunchKernelGGL(k_sample_cull, dim3((unsigned)nb), dim3(kBlock), 0, st, *geom, rays, total, n_words, bitmap,
+                       block_count, z_out);
+    LM_CHECK_LAUNCH("k_sample_cull");
+    hipLaunchKernelGGL(k_scan_blocks, dim3(1), dim3(1024), 0, st, (const uint32_t *)block_count, block_off,
+                       (uint32_t)nb, counters + LM_STAT_N_VALID);
+    LM_CHECK_LAUNCH("k_scan_blocks");
+    hipLaunchKernelGGL(k_emit, dim3((unsigned)nb), dim3(kBlock), 0, st, (const uint64_t *)bitmap, n_words,
+                       (const uint32_t *)block_off, word_prefix, valid_idx);
+    LM_CHECK_LAUNCH("k_emit");
+    return LM_OK;
+}

@@ -1,0 +1,413 @@
+"""Host-side mirror of the reference's render model on top of the C-ABI library.
+
+`GridNeRFHIP` keeps the call signature and the attributes callers read from the
+reference's `GridNeRF` in render mode (app/models/gridnerf_sequential.py:439-447 for
+`forward`; `run_nerf`, `alphaMask`, `aabb`, `n_importance`, `near_far`,
+`distance_scale`, `rayMarch_weight_thres`, `alpha_mask_filter_thre` as read by
+app/tools/render_utils.py:208 and dist_render/kernel/cuda_render_extend.py:43-159).
+PyTorch is used for device memory and streams only; every computation of the render
+path is a HIP kernel reached through ctypes.  There is no fallback: without the built
+library, or without a GPU, construction raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from types import SimpleNamespace
+from typing import Dict, Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib as L
+from .params import MAT_MODE, VEC_MODE, GridNeRFParams
+
+
+def _sampler_tables(p: GridNeRFParams, S: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-sample tables of the two samplers, evaluated with the same PyTorch CPU ops the
+    reference uses (gridnerf_sequential.py:268-273 and :303-304) so that they hold the
+    same bits: hull -> (near*(1-t), t) with t = linspace(0,1,S); aabb -> (stepSize*arange, 0)."""
+    if p.sampling_opt:
+        t = torch.linspace(0.0, 1.0, steps=S)
+        a = p.near_far[0] * (1.0 - t)
+    else:
+        t = torch.zeros(S)
+        a = (p.stepSize.cpu() * torch.arange(S)[None].float())[0]
+    return a.contiguous(), t.contiguous()
+
+
+class GridNeRFHIP:
+    """Render-only GridNeRF on one MI355X."""
+
+    def __init__(
+        self,
+        params: GridNeRFParams,
+        device: str = "cuda",
+        mlp_precision: str = "f32",
+        term_eps: float = 0.0,
+        release_source: bool = False,
+    ):
+        if not torch.cuda.is_available():
+            raise L.LandmarkError("GridNeRFHIP needs a GPU; there is no CPU path")
+        self.lib = L.load()
+        self.device = torch.device(device)
+        self.p = params
+        self.mlp_precision = mlp_precision
+        self.term_eps = float(term_eps)
+        if params.app_dim != 27 or params.view_pe != 2 or params.fea_pe != 2 or params.featureC != 128:
+            raise L.LandmarkError("colour network shape must be app_dim 27, view_pe = fea_pe = 2, featureC 128")
+        if params.fea2denseAct not in ("softplus", "relu"):
+            raise L.LandmarkError(f"fea2denseAct {params.fea2denseAct!r}")
+        # --- attributes the reference's callers read
+        self.run_nerf = False
+        self.aabb = params.aabb.to(self.device)
+        self.n_importance = params.n_importance
+        self.near_far = list(params.near_far)
+        self.distance_scale = params.distance_scale
+        self.rayMarch_weight_thres = params.rayMarch_weight_thres
+        self.alpha_mask_filter_thre = params.alpha_mask_filter_thre
+        self.sampling_opt = params.sampling_opt
+        self.ndims, self.resMode = params.ndims, list(params.resMode)
+        self.nSamples = params.nSamples
+        self.alphaMask = None
+        if params.alpha_volume is not None:
+            vol = params.alpha_volume.to(self.device, torch.float32).contiguous()
+            self.alphaMask = SimpleNamespace(
+                alpha_volume=vol.view(1, 1, *vol.shape[-3:]), aabb=params.alpha_aabb.to(self.device)
+            )
+        self._vol = None if self.alphaMask is None else self.alphaMask.alpha_volume
+        # --- channel-last tables
+        self._tables = []  # keep device tensors alive
+        self._density = self._relayout_set(params.density_plane, params.density_line)
+        self._app = self._relayout_set(params.app_plane, params.app_line)
+        self.K_app = sum(pl.C for pl in self._app)
+        if release_source:
+            params.density_plane, params.density_line, params.app_plane, params.app_line = [], [], [], []
+        # --- colour network
+        self._packed = {}
+        self._pack_mlp(mlp_precision)
+        # --- per-S geometry and workspace caches
+        self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
+        self._ws = None
+        self.counters = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)
+
+    # ------------------------------------------------------------------ construction helpers
+    def _relayout(self, t: torch.Tensor) -> torch.Tensor:
+        """[1,C,H,W] -> device [H,W,C] through lm_relayout_nchw_to_hwc."""
+        src = t.to(self.device).contiguous()
+        _, Cc, H, W = src.shape
+        dst = torch.empty((H, W, Cc), dtype=src.dtype, device=self.device)
+        dt = L.LM_F32 if src.dtype == torch.float32 else L.LM_F16
+        L.check(self.lib.lm_relayout_nchw_to_hwc(src.data_ptr(), dst.data_ptr(), Cc, H, W, dt, L.current_stream()), "relayout")
+        torch.cuda.current_stream().synchronize()  # src may be a temporary
+        return dst
+
+    def _relayout_set(self, planes, lines):
+        out = []
+        L_ = len(self.resMode)
+        if len(planes) > L.LM_MAX_PLANES:
+            raise L.LandmarkError(f"{len(planes)} planes > LM_MAX_PLANES")
+        for k, (pl, ln) in enumerate(zip(planes, lines)):
+            if pl.dtype not in (torch.float32, torch.float16):
+                raise L.LandmarkError(f"plane dtype {pl.dtype}")
+            P, Ln = self._relayout(pl), self._relayout(ln)
+            self._tables += [P, Ln]
+            d = k // L_
+            s = L.LmPlane()
+            s.plane, s.line = P.data_ptr(), Ln.data_ptr()
+            s.H, s.W, s.C = P.shape
+            s.Len = Ln.shape[0]
+            s.ax0, s.ax1 = MAT_MODE[d]
+            s.axl = VEC_MODE[d]
+            s.dtype = L.LM_F32 if P.dtype == torch.float32 else L.LM_F16
+            out.append(s)
+        return out
+
+    def _pack_mlp(self, precision: str):
+        if precision in self._packed:
+            return self._packed[precision]
+        prec = L.MLP_PREC[precision]
+        p = self.p
+        K = self.K_app
+        n = self.lib.lm_mlp_packed_bytes(prec, K)
+        if n == 0:
+            raise L.LandmarkError(self.lib.lm_last_error().decode())
+        host = np.zeros(n, dtype=np.uint8)
+        keep = []
+
+        def f(t):
+            if t is None:
+                return None
+            a = np.ascontiguousarray(t.detach().float().cpu().numpy())
+            keep.append(a)
+            return a.ctypes.data
+
+        L.check(
+            self.lib.lm_mlp_pack(
+                prec, K, f(p.basis_mat), f(p.mlp_w[0]), f(p.mlp_b[0]), f(p.mlp_w[1]), f(p.mlp_b[1]),
+                f(p.mlp_w[2]), f(p.mlp_b[2]), host.ctypes.data,
+            ),
+            "lm_mlp_pack",
+        )
+        dev = torch.from_numpy(host).to(self.device)
+        self._packed[precision] = (prec, dev)
+        return self._packed[precision]
+
+    def _geom(self, S: int) -> L.LmGeom:
+        if S in self._geom_cache:
+            return self._geom_cache[S][0]
+        p = self.p
+        a, t = _sampler_tables(p, S)
+        a_d, t_d = a.to(self.device), t.to(self.device)
+        g = L.LmGeom()
+        g.sampler = L.LM_SAMPLER_HULL if p.sampling_opt else L.LM_SAMPLER_AABB
+        g.S = S
+        g.aabb[:] = p.aabb.detach().cpu().reshape(-1).tolist()
+        g.near_ = torch.tensor(p.near_far[0], dtype=torch.float32).item()
+        g.far_ = torch.tensor(p.near_far[1], dtype=torch.float32).item()
+        g.tab_a, g.tab_t = a_d.data_ptr(), t_d.data_ptr()
+        g.inv_aabb[:] = p.invaabbSize.detach().cpu().tolist()
+        if self._vol is not None:
+            g.vol = self._vol.data_ptr()
+            g.vd, g.vh, g.vw = self._vol.shape[-3:]
+            ab = p.alpha_aabb.detach().cpu()
+            g.vol_aabb_min[:] = ab[0].tolist()
+            g.vol_inv[:] = (1.0 / (ab[1] - ab[0]) * 2).tolist()
+            g.vol_thre = torch.tensor(p.alpha_mask_filter_thre, dtype=torch.float32).item()
+        self._geom_cache[S] = (g, (a_d, t_d))
+        return g
+
+    def _model_struct(self, S: int, white_bg: bool) -> L.LmModel:
+        m = L.LmModel()
+        m.geom = self._geom(S)
+        m.n_planes = len(self._density)
+        for k in range(len(self._density)):
+            m.density[k] = self._density[k]
+            m.app[k] = self._app[k]
+        m.act = L.LM_ACT_SOFTPLUS if self.p.fea2denseAct == "softplus" else L.LM_ACT_RELU
+        m.density_shift = self.p.density_shift
+        m.distance_scale = self.p.distance_scale
+        m.weight_thres = self.p.rayMarch_weight_thres
+        prec, packed = self._pack_mlp(self.mlp_precision)
+        m.mlp_prec, m.mlp_packed = prec, packed.data_ptr()
+        m.white_bg = int(bool(white_bg))
+        m.term_eps = self.term_eps
+        return m
+
+    def _samples_for(self, N_samples: int) -> int:
+        if self.p.sampling_opt:
+            return int(self.p.n_importance)
+        return int(N_samples) if N_samples > 0 else int(self.nSamples)
+
+    def workspace(self, n_rays: int, S: int) -> torch.Tensor:
+        """Device workspace for chunks of up to n_rays rays; grown on demand and reused
+        (the role of allocate_tensors, dist_render/kernel/cuda_render_extend.py:35-159)."""
+        need = self.lib.lm_render_workspace_bytes(n_rays, S, self.K_app)
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = None
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return self._ws
+
+    # ------------------------------------------------------------------ reference interface
+    def eval(self):
+        return self
+
+    def to(self, device):
+        return self
+
+    @torch.no_grad()
+    def forward(self, rays_chunk, app_code=None, white_bg=True, is_train=False, N_samples=-1, idxs_chunk=None):
+        """GridBaseSequential.forward in render mode -> ({"rgb_map","depth_map"}, {})."""
+        if is_train:
+            raise NotImplementedError("training is outside this render path (is_train must be False)")
+        if app_code is not None or idxs_chunk is not None:
+            raise NotImplementedError("appearance embedding (encode_app) is not part of this render path")
+        rays = rays_chunk.to(self.device, torch.float32).contiguous()
+        if rays.dim() != 2 or rays.shape[1] != 6:
+            raise ValueError(f"rays_chunk must be [N,6], got {tuple(rays.shape)}")
+        N = rays.shape[0]
+        S = self._samples_for(N_samples)
+        rgb = torch.empty((N, 3), dtype=torch.float32, device=self.device)
+        depth = torch.empty((N,), dtype=torch.float32, device=self.device)
+        if N:
+            ws = self.workspace(N, S)
+            m = self._model_struct(S, white_bg)
+            L.check(
+                self.lib.lm_render(
+                    C.byref(m), rays.data_ptr(), N, ws.data_ptr(), ws.numel(), rgb.data_ptr(), depth.data_ptr(),
+                    self.counters.data_ptr(), L.current_stream(),
+                ),
+                "lm_render",
+            )
+        return {"rgb_map": rgb, "depth_map": depth}, {}
+
+    __call__ = forward
+
+    def last_counts(self) -> Dict[str, int]:
+        """Valid / appearance sample counts of the last chunk (synchronises)."""
+        c = self.counters.cpu()
+        return {"n_valid": int(c[L.LM_STAT_N_VALID]) & 0xFFFFFFFF, "n_app": int(c[L.LM_STAT_N_APP]) & 0xFFFFFFFF}
+
+    # ------------------------------------------------------------------ stage entry points
+    @torch.no_grad()
+    def sample_cull(self, rays, N_samples=-1, want_z=True):
+        """Part 1 alone: valid mask [N,S], ascending valid flat indices, depths."""
+        rays = rays.to(self.device, torch.float32).contiguous()
+        N, S = rays.shape[0], self._samples_for(N_samples)
+        total = N * S
+        n_words = (total + 63) // 64
+        bitmap = torch.zeros(max(n_words, 1), dtype=torch.int64, device=self.device)
+        prefix = torch.zeros(max(n_words, 1), dtype=torch.int32, device=self.device)
+        idx = torch.empty(max(total, 1), dtype=torch.int32, device=self.device)
+        z = torch.empty((N, S), dtype=torch.float32, device=self.device) if want_z else None
+        scratch = torch.empty(max(self.lib.lm_sample_cull_scratch_bytes(N, S), 256), dtype=torch.uint8, device=self.device)
+        cnt = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)
+        g = self._geom(S)
+        L.check(
+            self.lib.lm_sample_cull(
+                C.byref(g), rays.data_ptr(), N, bitmap.data_ptr(), prefix.data_ptr(), idx.data_ptr(), cnt.data_ptr(),
+                L.ptr(z), scratch.data_ptr(), L.current_stream(),
+            ),
+            "lm_sample_cull",
+        )
+        n_valid = int(cnt[L.LM_STAT_N_VALID].item()) & 0xFFFFFFFF
+        bits = (bitmap[:, None] >> torch.arange(64, device=self.device)) & 1
+        mask = bits.reshape(-1)[:total].bool().view(N, S)
+        return {
+            "ray_valid": mask, "valid_idx": idx[:n_valid].long() & 0xFFFFFFFF, "n_valid": n_valid, "z_vals": z,
+            "bitmap": bitmap, "word_prefix": prefix, "counters": cnt, "valid_idx_raw": idx, "rays": rays, "S": S,
+        }
+
+    def _plane_array(self, planes):
+        arr = (L.LmPlane * len(planes))()
+        for k, s in enumerate(planes):
+            arr[k] = s
+        return arr
+
+    @torch.no_grad()
+    def compute_densityfeature(self, xyz_sampled):
+        """GridNeRF.compute_densityfeature on normalised coordinates [M,3] -> [M]."""
+        xyz = xyz_sampled.to(self.device, torch.float32).contiguous()
+        M = xyz.shape[0]
+        out = torch.empty(M, dtype=torch.float32, device=self.device)
+        arr = self._plane_array(self._density)
+        L.check(self.lib.lm_gather_density_xyz(arr, len(self._density), xyz.data_ptr(), M, out.data_ptr(), L.current_stream()), "lm_gather_density_xyz")
+        return out
+
+    @torch.no_grad()
+    def app_products(self, xyz_sampled):
+        """plane*line products [M, P*L*C_a] (compute_appfeature before basis_mat)."""
+        xyz = xyz_sampled.to(self.device, torch.float32).contiguous()
+        M = xyz.shape[0]
+        out = torch.empty((M, self.K_app), dtype=torch.float32, device=self.device)
+        arr = self._plane_array(self._app)
+        L.check(self.lib.lm_gather_app_xyz(arr, len(self._app), xyz.data_ptr(), M, out.data_ptr(), L.current_stream()), "lm_gather_app_xyz")
+        return out
+
+    @torch.no_grad()
+    def basis(self, products, precision=None):
+        prec, packed = self._pack_mlp(precision or self.mlp_precision)
+        products = products.to(self.device, torch.float32).contiguous()
+        M = products.shape[0]
+        out = torch.empty((M, 27), dtype=torch.float32, device=self.device)
+        L.check(self.lib.lm_basis(prec, packed.data_ptr(), self.K_app, products.data_ptr(), M, out.data_ptr(), L.current_stream()), "lm_basis")
+        return out
+
+    @torch.no_grad()
+    def compute_appfeature(self, xyz_sampled, precision=None):
+        """GridNeRF.compute_appfeature: basis_mat(products) -> [M,27]."""
+        return self.basis(self.app_products(xyz_sampled), precision)
+
+    @torch.no_grad()
+    def render_module(self, viewdirs, features, precision=None):
+        """MLPRender_Fea.forward(viewdirs, features) -> rgb [M,3]."""
+        prec, packed = self._pack_mlp(precision or self.mlp_precision)
+        feat = features.to(self.device, torch.float32).contiguous()
+        view = viewdirs.to(self.device, torch.float32).contiguous()
+        M = feat.shape[0]
+        out = torch.empty((M, 3), dtype=torch.float32, device=self.device)
+        L.check(self.lib.lm_mlp(prec, packed.data_ptr(), self.K_app, feat.data_ptr(), view.data_ptr(), M, out.data_ptr(), L.current_stream()), "lm_mlp")
+        return out
+
+    renderModule = render_module
+
+    @torch.no_grad()
+    def density_valid(self, cull, white_bg=True):
+        """sigma of the valid samples of a `sample_cull` result, in list order."""
+        m = self._model_struct(cull["S"], white_bg)
+        sigma = torch.zeros(max(cull["n_valid"], 1), dtype=torch.float32, device=self.device)
+        L.check(
+            self.lib.lm_density_valid(C.byref(m), cull["rays"].data_ptr(), cull["valid_idx_raw"].data_ptr(), cull["counters"].data_ptr(), sigma.data_ptr(), L.current_stream()),
+            "lm_density_valid",
+        )
+        return sigma[: cull["n_valid"]]
+
+    @torch.no_grad()
+    def weights(self, cull, sigma, term_eps=None):
+        """Part 4 on a `sample_cull` result: dense weights, appearance mask, acc, depth."""
+        rays, S = cull["rays"], cull["S"]
+        N = rays.shape[0]
+        steps = (S + 63) // 64
+        dev = self.device
+        weight = torch.zeros((N, S), dtype=torch.float32, device=dev)
+        app_bits = torch.zeros((N, steps), dtype=torch.int64, device=dev)
+        app_base = torch.zeros((N, steps), dtype=torch.int32, device=dev)
+        app_idx = torch.zeros(max(N * S, 1), dtype=torch.int32, device=dev)
+        app_w = torch.zeros(max(N * S, 1), dtype=torch.float32, device=dev)
+        acc = torch.zeros(N, dtype=torch.float32, device=dev)
+        depth = torch.zeros(N, dtype=torch.float32, device=dev)
+        cnt = cull["counters"].clone()
+        cnt[L.LM_STAT_N_APP] = 0
+        sig = sigma if sigma.numel() else torch.zeros(1, device=dev)
+        g = self._geom(S)
+        L.check(
+            self.lib.lm_weights(
+                C.byref(g), rays.data_ptr(), N, cull["bitmap"].data_ptr(), cull["word_prefix"].data_ptr(), sig.data_ptr(),
+                self.p.distance_scale, self.p.rayMarch_weight_thres, self.term_eps if term_eps is None else term_eps,
+                weight.data_ptr(), app_bits.data_ptr(), app_base.data_ptr(), app_idx.data_ptr(), app_w.data_ptr(),
+                acc.data_ptr(), depth.data_ptr(), cnt.data_ptr(), L.current_stream(),
+            ),
+            "lm_weights",
+        )
+        n_app = int(cnt[L.LM_STAT_N_APP].item()) & 0xFFFFFFFF
+        bits = (app_bits[:, :, None] >> torch.arange(64, device=dev)) & 1
+        app_mask = bits.reshape(N, steps * 64)[:, :S].bool()
+        return {
+            "weight": weight, "app_mask": app_mask, "acc_map": acc, "depth_map": depth, "n_app": n_app,
+            "app_idx": app_idx[:n_app].long() & 0xFFFFFFFF, "app_w": app_w[:n_app],
+        }
+
+
+def from_reference_model(model, **kw) -> GridNeRFHIP:
+    """Build from an object with the reference model's attributes (a loaded
+    `GridNeRF`, gridnerf_sequential.py:661-747) without importing the reference."""
+    lin = [model.renderModule.mlp[i] for i in (0, 2, 4)]
+    am = getattr(model, "alphaMask", None)
+    p = GridNeRFParams(
+        aabb=model.aabb.detach().float().cpu(),
+        gridSize=[int(x) for x in model.gridSize.tolist()],
+        density_plane=[t.detach() for t in model.density_plane],
+        density_line=[t.detach() for t in model.density_line],
+        app_plane=[t.detach() for t in model.app_plane],
+        app_line=[t.detach() for t in model.app_line],
+        basis_mat=model.basis_mat.weight.detach(),
+        mlp_w=[l.weight.detach() for l in lin],
+        mlp_b=[None if l.bias is None else l.bias.detach() for l in lin],
+        ndims=model.ndims,
+        resMode=list(model.resMode),
+        near_far=[float(x) for x in model.near_far],
+        density_shift=float(model.density_shift),
+        distance_scale=float(model.distance_scale),
+        rayMarch_weight_thres=float(model.rayMarch_weight_thres),
+        fea2denseAct=model.fea2denseAct,
+        step_ratio=float(model.step_ratio),
+        sampling_opt=int(model.sampling_opt),
+        n_importance=int(model.n_importance),
+        view_pe=model.view_pe,
+        fea_pe=model.fea_pe,
+        app_dim=model.app_dim,
+        featureC=model.featureC,
+        alpha_volume=None if am is None else am.alpha_volume[0, 0].detach(),
+        alpha_aabb=None if am is None else am.aabb.detach().cpu(),
+        alpha_mask_filter_thre=float(model.alpha_mask_filter_thre),
+    )
+    return GridNeRFHIP(p, **kw)

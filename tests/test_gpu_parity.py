@@ -1,0 +1,262 @@
+"""GPU parity tests: the HIP path through the C-ABI against the CPU oracle.
+
+Bars (BASELINE north star): sample masks, sample counts and valid-sample indices
+bit-exact; depths of the samples bit-exact; rgb / depth within 1e-4 absolute with fp32
+tables and an fp32 colour network, 1e-2 with fp16 tables or a 16-bit colour network.
+The appearance mask (weight > 1e-3) derives from floats that are summed in a different
+order than ATen does, so it may flip for weights within rounding of the threshold; such
+samples are excluded by an explicit band and counted.
+"""
+import pytest
+import torch
+
+from landmark_amd import scenes
+from oracle import gridnerf_oracle as O
+from tests.helpers import golden_names, load_golden
+
+pytestmark = pytest.mark.gpu
+
+RGB_TOL_F32 = 1e-4
+RGB_TOL_16 = 1e-2
+
+
+def _model(p, **kw):
+    from landmark_amd.model import GridNeRFHIP
+
+    return GridNeRFHIP(p, **kw)
+
+
+def _scene(seed=3, grid=(9, 11, 13), opt=1, S=64, with_mask=True, thre=0.0, shift=0.0, boost=6.0, **kw):
+    p = scenes.make_params(seed=seed, gridSize=grid, near_far=[0.5, 4.5], n_importance=S, sampling_opt=opt,
+                           density_shift=shift, **kw)
+    for t in p.density_plane:
+        t.mul_(boost)
+    if with_mask:
+        p.alpha_volume = scenes.blob_occupancy((grid[2], grid[1], grid[0]), 6, 0.45, seed=seed)
+        p.alpha_aabb = p.aabb + torch.tensor([[0.01, 0.0, -0.02], [0.0, 0.05, 0.0]])
+        p.alpha_mask_filter_thre = thre
+    return p
+
+
+# ------------------------------------------------------------------------------------ part 1
+@pytest.mark.parametrize("name", golden_names())
+def test_sample_cull_golden(gpu_lib, name):
+    p, d, cfg = load_golden(name)
+    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], return_aux=True)
+    out = _model(p).sample_cull(d["rays"], N_samples=cfg["N_samples"])
+    assert torch.equal(out["z_vals"].cpu(), ref["z_vals"])
+    assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
+    assert out["n_valid"] == int(ref["ray_valid"].sum())
+    assert torch.equal(out["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
+
+
+@pytest.mark.parametrize("opt,S,thre", [(1, 64, 0.0), (1, 128, 0.5), (1, 100, 0.98), (0, 50, 0.0), (0, 77, 0.5)])
+def test_sample_cull_random_scene_bit_exact(gpu_lib, opt, S, thre):
+    p = _scene(opt=opt, S=S, thre=thre, step_ratio=0.4)
+    rays = scenes.pinhole_rays(96, 96, 80.0, scenes.sphere_pose(2.5, 5))
+    ref = O.render_chunk(p, rays, N_samples=S, return_aux=True)
+    out = _model(p).sample_cull(rays, N_samples=S)
+    assert 0 < int(ref["ray_valid"].sum()) < ref["ray_valid"].numel()
+    assert torch.equal(out["z_vals"].cpu(), ref["z_vals"])
+    assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
+    assert torch.equal(out["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
+
+
+def test_sample_cull_edge_cases(gpu_lib):
+    p = _scene(with_mask=False, S=64)
+    m = _model(p)
+    # empty chunk
+    out = m.sample_cull(torch.zeros(0, 6))
+    assert out["n_valid"] == 0
+    # every ray misses the box -> empty list
+    rays = torch.tensor([[5.0, 5.0, 5.0, 0.0, 0.0, 1.0]]).repeat(70, 1)
+    out = m.sample_cull(rays)
+    assert out["n_valid"] == 0 and not out["ray_valid"].any()
+    # one ray, ragged tail (N*S not a multiple of a 4096-sample workgroup)
+    rays = scenes.pinhole_rays(3, 1, 4.0, scenes.sphere_pose(2.5, 1))
+    ref = O.render_chunk(p, rays, return_aux=True)
+    out = m.sample_cull(rays)
+    assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
+    # all-ones occupancy keeps every in-box sample, all-zeros none
+    p.alpha_volume, p.alpha_aabb = torch.ones(4, 4, 4), p.aabb.clone()
+    assert _model(p).sample_cull(rays)["n_valid"] == int(ref["ray_valid"].sum())
+    p.alpha_volume = torch.zeros(4, 4, 4)
+    assert _model(p).sample_cull(rays)["n_valid"] == 0
+
+
+# ------------------------------------------------------------------------------------ part 2
+@pytest.mark.parametrize("ndims,res,dn,an", [(3, (1,), 16, 48), (1, (1, 2, 4), 16, 48), (3, (1, 2), 64, 64), (2, (1,), 8, 12)])
+def test_gather_matches_grid_sample(gpu_lib, ndims, res, dn, an):
+    p = scenes.make_params(seed=7, gridSize=(13, 9, 11), ndims=ndims, resMode=res, density_n_comp=dn, app_n_comp=an,
+                           feature_init="uniform")
+    g = torch.Generator().manual_seed(8)
+    xyz = torch.rand(5000, 3, generator=g) * 2.2 - 1.1  # a band outside [-1,1] exercises zero padding
+    xyz[:8] = torch.tensor([[-1.0, -1, -1], [1, 1, 1], [1, -1, 0], [0, 0, 0], [-1, 1, 1], [0.5, 1, -1], [1, 0.25, 1], [-1, -1, 1]])
+    m = _model(p)
+    ref_d = O.density_feature(p, xyz)
+    assert torch.allclose(m.compute_densityfeature(xyz).cpu(), ref_d, atol=2e-5 * max(1, dn // 16 * len(res) * ndims))
+    ref_a = O.app_products(p, xyz)
+    got_a = m.app_products(xyz).cpu()
+    assert got_a.shape == ref_a.shape
+    assert torch.allclose(got_a, ref_a, atol=2e-6)
+
+
+def test_gather_fp16_tables(gpu_lib):
+    p = scenes.make_params(seed=9, gridSize=(17, 12, 10), ndims=3, resMode=(1, 2), density_n_comp=16, app_n_comp=48,
+                           dtype=torch.float16)
+    g = torch.Generator().manual_seed(8)
+    xyz = torch.rand(4000, 3, generator=g) * 2 - 1
+    m = _model(p)
+    # the oracle interpolates the same fp16 values in fp32, so only summation order differs
+    assert torch.allclose(m.compute_densityfeature(xyz).cpu(), O.density_feature(p, xyz), atol=2e-5)
+    assert torch.allclose(m.app_products(xyz).cpu(), O.app_products(p, xyz), atol=2e-6)
+
+
+def test_gather_closed_forms(gpu_lib):
+    p = scenes.make_params(seed=1, gridSize=(7, 5, 9), density_n_comp=16, app_n_comp=48, ndims=3, resMode=(1, 2))
+    for k, pl in enumerate(p.density_plane):
+        H, W = pl.shape[-2:]
+        ys, xs = torch.meshgrid(torch.linspace(-1, 1, H), torch.linspace(-1, 1, W), indexing="ij")
+        pl.zero_()
+        pl[0, 3] = (0.3 + 0.1 * k) * xs + (-0.2 + 0.05 * k) * ys + 0.7
+        p.density_line[k].fill_(1.0)
+    g = torch.Generator().manual_seed(2)
+    xyz = torch.rand(300, 3, generator=g) * 2 - 1
+    exp = torch.zeros(300)
+    for k in range(6):
+        m0, m1 = O.MAT_MODE[k // 2]
+        exp += (0.3 + 0.1 * k) * xyz[:, m0] + (-0.2 + 0.05 * k) * xyz[:, m1] + 0.7
+    assert torch.allclose(_model(p).compute_densityfeature(xyz).cpu(), exp, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------ part 3
+@pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16", 4e-3), ("bf16", 3e-2)])
+def test_colour_network(gpu_lib, prec, tol):
+    p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48)
+    g = torch.Generator().manual_seed(6)
+    for M in (1, 31, 32, 33, 4097):
+        feats, view = torch.randn(M, 27, generator=g), torch.randn(M, 3, generator=g)
+        got = _model(p).render_module(view, feats, precision=prec).cpu()
+        ref = O.mlp_render(p, view, feats)
+        assert (got - ref).abs().max().item() < tol, (M, prec)
+
+
+@pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16", 2e-3)])
+def test_basis_projection(gpu_lib, prec, tol):
+    p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48, ndims=3, resMode=(1, 2))
+    g = torch.Generator().manual_seed(6)
+    prod = torch.randn(1000, 288, generator=g)
+    got = _model(p).basis(prod, precision=prec).cpu()
+    assert (got - O.F.linear(prod, p.basis_mat)).abs().max().item() < tol
+    onehot = torch.zeros(3, 288)
+    onehot[0, 5], onehot[1, 48 + 7], onehot[2, 287] = 1, 1, 1
+    got = _model(p).basis(onehot, precision="f32").cpu()
+    assert torch.allclose(got, p.basis_mat[:, [5, 55, 287]].T, atol=1e-7)
+
+
+# ------------------------------------------------------------------------------------ part 4
+def test_weights_against_raw2alpha(gpu_lib):
+    p = _scene(S=128, thre=0.0)
+    rays = scenes.pinhole_rays(64, 64, 60.0, scenes.sphere_pose(2.5, 5))
+    ref = O.render_chunk(p, rays, return_aux=True)
+    m = _model(p)
+    cull = m.sample_cull(rays)
+    sigma = m.density_valid(cull)
+    assert torch.allclose(sigma.cpu(), ref["sigma"][ref["ray_valid"]], atol=2e-5, rtol=1e-5)
+    w = m.weights(cull, sigma)
+    assert torch.allclose(w["weight"].cpu(), ref["weight"], atol=1e-5)
+    assert torch.allclose(w["acc_map"].cpu(), ref["acc_map"], atol=1e-5)
+    assert torch.allclose(w["depth_map"].cpu(), ref["depth_map"], atol=2e-5)
+    band = (ref["weight"] - p.rayMarch_weight_thres).abs() < 1e-6
+    assert torch.equal(w["app_mask"].cpu() | band, ref["app_mask"] | band)
+    assert w["n_app"] == int(w["app_mask"].sum())
+    # the appearance list holds exactly the masked samples, each with its weight
+    flat = w["app_mask"].reshape(-1).nonzero()[:, 0]
+    order = torch.argsort(w["app_idx"])
+    assert torch.equal(w["app_idx"][order], flat)
+    assert torch.equal(w["app_w"][order], w["weight"].reshape(-1)[flat])
+
+
+# ------------------------------------------------------------------------------------ whole path
+def _check_render(p, rays, tol, S=-1, white_bg=True, **kw):
+    ref = O.render_chunk(p, rays, white_bg=white_bg, N_samples=S, return_aux=True)
+    out, extra = _model(p, **kw)(rays, white_bg=white_bg, N_samples=S)
+    assert extra == {} and set(out) == {"rgb_map", "depth_map"}
+    # rays holding a sample whose weight sits within rounding of the threshold may differ by that sample
+    band = ((ref["weight"] - p.rayMarch_weight_thres).abs() < 2e-6).any(-1)
+    ok = ~band
+    d_rgb = (out["rgb_map"].cpu() - ref["rgb_map"]).abs().max(-1).values
+    d_dep = (out["depth_map"].cpu() - ref["depth_map"]).abs()
+    assert d_rgb[ok].max().item() <= tol, f"rgb max diff {d_rgb[ok].max().item()}"
+    assert d_dep[ok].max().item() <= tol, f"depth max diff {d_dep[ok].max().item()}"
+    assert int(band.sum()) <= max(2, rays.shape[0] // 2000)
+    if band.any():
+        assert d_rgb[band].max().item() <= 2e-3
+    return ref, out
+
+
+@pytest.mark.parametrize("name", golden_names())
+def test_render_golden_vectors(gpu_lib, name):
+    p, d, cfg = load_golden(name)
+    out, _ = _model(p)(d["rays"], white_bg=True, N_samples=cfg["N_samples"])
+    assert (out["rgb_map"].cpu() - d["rgb_map"]).abs().max().item() <= RGB_TOL_F32
+    assert (out["depth_map"].cpu() - d["depth_map"]).abs().max().item() <= RGB_TOL_F32
+    out, _ = _model(p)(d["rays"], white_bg=False, N_samples=cfg["N_samples"])
+    assert (out["rgb_map"].cpu() - d["rgb_map_black"]).abs().max().item() <= RGB_TOL_F32
+
+
+@pytest.mark.parametrize("opt,act,shift,res,ndims", [(1, "softplus", 0.0, (1,), 3), (1, "relu", -10.0, (1, 2, 4), 1), (0, "softplus", -1.0, (1, 2), 3)])
+def test_render_random_scenes(gpu_lib, opt, act, shift, res, ndims):
+    p = _scene(opt=opt, S=128, shift=shift, fea2denseAct=act, resMode=res, ndims=ndims, step_ratio=0.3, thre=0.0)
+    rays = scenes.pinhole_rays(80, 80, 70.0, scenes.sphere_pose(2.5, 9))
+    ref, _ = _check_render(p, rays, RGB_TOL_F32, S=128)
+    assert ref["app_mask"].any(), "scene must exercise the colour network"
+
+
+def test_render_c1_tiny_config(gpu_lib):
+    """BASELINE config 1 at reduced image size (the oracle finishes in seconds): the stated
+    init (background only) and the dense variant that runs every stage."""
+    rays = scenes.c1_rays(64, 64)
+    for dense in (False, True):
+        p = scenes.c1_scene(dense=dense)
+        ref, _ = _check_render(p, rays, RGB_TOL_F32)
+        assert bool(ref["app_mask"].any()) == dense
+
+
+def test_render_16bit_network_and_fp16_tables(gpu_lib):
+    p = _scene(S=64)
+    rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    _check_render(p, rays, RGB_TOL_16, mlp_precision="f16")
+    _check_render(p, rays, 3e-2, mlp_precision="bf16")
+    _check_render(O.to_fp16_features(p), rays, RGB_TOL_16)
+
+
+def test_chunk_drivers(gpu_lib):
+    from landmark_amd.render import MultiBlockParallelHIP, renderer_fn
+
+    p = _scene(S=64)
+    rays = scenes.pinhole_rays(40, 40, 40.0, scenes.sphere_pose(2.5, 5))
+    m = _model(p)
+    full, _ = m(rays)
+    for chunk in (1, 333, 4096):
+        ret, extra = renderer_fn(rays, m, chunk=chunk, device="cuda")
+        assert extra == {} and set(ret) == {"rgb_map", "depth_map"}
+        # rays are independent: any chunking gives identical bits
+        assert torch.equal(ret["rgb_map"], full["rgb_map"]) and torch.equal(ret["depth_map"], full["depth_map"])
+    fused = MultiBlockParallelHIP()
+    fused.allocate_tensors(m, 512)
+    ret = fused.forward(rays[:512].cuda(), app_code=None, white_bg=True)
+    assert torch.equal(ret["rgb_map"], full["rgb_map"][:512])
+    with pytest.raises(NotImplementedError):
+        m(rays, is_train=True)
+
+
+def test_early_termination_bounds(gpu_lib):
+    p = _scene(S=128)
+    rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    exact, _ = _model(p)(rays)
+    term, _ = _model(p, term_eps=1e-4)(rays)
+    # all samples after T < 1e-4 have weight < 1e-4 < threshold: colour unchanged up to the white
+    # background term (<= 1e-4); depth loses at most T * z_far
+    assert (term["rgb_map"] - exact["rgb_map"]).abs().max().item() <= 1e-4
+    assert (term["depth_map"] - exact["depth_map"]).abs().max().item() <= 1e-4 * 4.5 * 1.5

@@ -1,0 +1,145 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol
+the header declares, argument validation works, and the weight packing of the colour
+network reproduces the oracle when replayed through a numpy model of the matrix-core
+data flow (32x32 accumulator layout: lane l -> column l%32, register v -> row
+8*(v/4) + 4*(l/32) + v%4)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from landmark_amd import _lib as L
+from landmark_amd import scenes
+from oracle import gridnerf_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(L.SO_PATH):
+        from landmark_amd import build
+
+        build.build(verbose=False)
+    return L.load()
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = open(os.path.join(ROOT, "include", "landmark_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(lm_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    assert declared == set(L.SYMBOLS), f"binding table and header differ: {declared ^ set(L.SYMBOLS)}"
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_struct_sizes_match_header_layout():
+    assert C.sizeof(L.LmPlane) == 48
+    assert C.sizeof(L.LmGeom) == 4 * 2 + 24 + 8 + 16 + 12 + 4 + 8 + 12 + 12 + 12 + 4
+    assert C.sizeof(L.LmModel) % 8 == 0
+
+
+def test_argument_validation_returns_status_not_abort(lib):
+    g = L.LmGeom()
+    g.S = 0
+    rc = lib.lm_sample_cull(C.byref(g), None, 4, None, None, None, None, None, None, None)
+    assert rc == -1 and b"S must be positive" in lib.lm_last_error()
+    assert lib.lm_mlp_packed_bytes(7, 144) == 0
+    assert lib.lm_mlp_packed_bytes(L.LM_MLP_F32, 100) == 0  # K not a multiple of 16
+    assert lib.lm_render_workspace_bytes(0, 128, 144) == 0
+    pl = (L.LmPlane * 1)()
+    rc = lib.lm_gather_density_xyz(pl, 1, None, 10, None, None)
+    assert rc == -1 and b"null table" in lib.lm_last_error()
+    assert lib.lm_gather_density_xyz(pl, 13, None, 10, None, None) == -1
+    assert lib.lm_relayout_nchw_to_hwc(None, None, 4, 4, 4, 0, None) == -1
+
+
+def test_workspace_size_grows_with_chunk(lib):
+    a = lib.lm_render_workspace_bytes(1024, 128, 144)
+    b = lib.lm_render_workspace_bytes(2048, 128, 144)
+    c = lib.lm_render_workspace_bytes(2048, 128, 432)
+    assert 0 < a < b < c
+
+
+# ---------------------------------------------------------------- packing replay
+def row_of(v, h):
+    return 8 * (v // 4) + 4 * h + v % 4
+
+
+def _layout(prec, K):
+    E = 4 if prec == L.LM_MLP_F32 else 2
+    al = lambda x: (x + 255) & ~255
+    o = 0
+    out = {}
+    for name, n in (("basis", 32 * K * E), ("w1", 4 * 80 * 64 * E), ("b1", 512), ("w2", 4 * 64 * 64 * E), ("b2", 512), ("w3", 64 * 64 * E), ("b3", 128)):
+        out[name] = o
+        o = al(o + n)
+    out["total"] = o
+    return out
+
+
+def _frags(buf, off, n_blocks, n_slots, G, dt):
+    steps = n_slots // G
+    n = n_blocks * steps * 64 * G
+    a = np.frombuffer(buf, dtype=dt, count=n, offset=off).astype(np.float32)
+    return a.reshape(n_blocks, steps, 64, G)
+
+
+def _mma_layer(A, slots):
+    """A: [nb, steps, 64, G] fragments; slots: [n_samples, 2(h), n_slots] -> D [n_samples, nb, 32 rows]"""
+    nb, steps, _, G = A.shape
+    Ar = A.reshape(nb, steps, 2, 32, G)  # lane = h*32 + i
+    sl = slots.reshape(slots.shape[0], 2, steps, G)
+    return np.einsum("bthig,nhtg->nbi", Ar.astype(np.float64), sl.astype(np.float64))
+
+
+def _regs(D):
+    """D [n, nb, 32] -> per-lane-half registers [n, 2, nb*16] (v = 0..15 per block)"""
+    n, nb, _ = D.shape
+    out = np.zeros((n, 2, nb, 16))
+    for h in range(2):
+        for v in range(16):
+            out[:, h, :, v] = D[:, :, row_of(v, h)]
+    return out.reshape(n, 2, nb * 16)
+
+
+@pytest.mark.parametrize("prec,dt,tol", [(L.LM_MLP_F32, np.float32, 2e-6), (L.LM_MLP_F16, np.float16, 3e-3)])
+def test_packed_weights_replay_matches_oracle(lib, prec, dt, tol):
+    p = scenes.make_params(seed=11, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=16, ndims=3, resMode=(1,))
+    K = 48
+    n = lib.lm_mlp_packed_bytes(prec, K)
+    lay = _layout(prec, K)
+    assert n == lay["total"]
+    host = np.zeros(n, np.uint8)
+    arrs = [np.ascontiguousarray(t.numpy()) for t in (p.basis_mat, p.mlp_w[0], p.mlp_b[0], p.mlp_w[1], p.mlp_b[1], p.mlp_w[2], p.mlp_b[2])]
+    rc = lib.lm_mlp_pack(prec, K, *[a.ctypes.data for a in arrs], host.ctypes.data)
+    assert rc == 0
+    buf = host.tobytes()
+    G = 1 if prec == L.LM_MLP_F32 else 8
+    CW = 4 if prec == L.LM_MLP_F32 else 8
+    g = torch.Generator().manual_seed(1)
+    ns = 37
+    prod = torch.randn(ns, K, generator=g)
+    view = torch.randn(ns, 3, generator=g)
+    # basis: lane-half h reads channels 2W*(s/W) + W*h + s%W
+    ch = np.array([[2 * CW * (s // CW) + CW * h + s % CW for s in range(K // 2)] for h in range(2)])
+    slots = prod.numpy()[:, ch]  # [n, 2, K/2]
+    feat_rows = _mma_layer(_frags(buf, lay["basis"], 1, K // 2, G, dt), slots)  # [n,1,32]
+    ref_feat = O.F.linear(prod, p.basis_mat).numpy()
+    assert np.allclose(feat_rows[:, 0, :27], ref_feat, atol=tol * 10)
+    assert np.all(feat_rows[:, 0, 27:] == 0)
+    raw = _regs(feat_rows)  # [n,2,16]
+    raw[:, 1, 12:15] = view.numpy()
+    raw[:, :, 15] = 0
+    s1 = np.concatenate([raw, np.sin(raw), np.cos(raw), np.sin(2 * raw), np.cos(2 * raw)], axis=2)  # [n,2,80]
+    bias = lambda name, nb: np.frombuffer(buf, np.float32, nb * 32, lay[name]).reshape(nb, 2, 16)
+    h1 = np.maximum(_regs(_mma_layer(_frags(buf, lay["w1"], 4, 80, G, dt), s1)) + bias("b1", 4).transpose(1, 0, 2).reshape(2, 64), 0)
+    h2 = np.maximum(_regs(_mma_layer(_frags(buf, lay["w2"], 4, 64, G, dt), h1)) + bias("b2", 4).transpose(1, 0, 2).reshape(2, 64), 0)
+    o = _regs(_mma_layer(_frags(buf, lay["w3"], 1, 64, G, dt), h2)) + bias("b3", 1).transpose(1, 0, 2).reshape(2, 16)
+    rgb = 1 / (1 + np.exp(-o[:, 0, :3]))
+    ref = O.mlp_render(p, view, torch.from_numpy(ref_feat)).numpy()
+    assert np.allclose(rgb, ref, atol=tol)
