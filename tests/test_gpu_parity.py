@@ -85,7 +85,7 @@ def test_sample_cull_edge_cases(gpu_lib):
 
 
 # ------------------------------------------------------------------------------------ part 2
-@pytest.mark.parametrize("ndims,res,dn,an", [(3, (1,), 16, 48), (1, (1, 2, 4), 16, 48), (3, (1, 2), 64, 64), (2, (1,), 8, 12)])
+@pytest.mark.parametrize("ndims,res,dn,an", [(3, (1,), 16, 48), (1, (1, 2, 4), 16, 48), (3, (1, 2), 64, 64), (2, (1,), 8, 16)])
 def test_gather_matches_grid_sample(gpu_lib, ndims, res, dn, an):
     p = scenes.make_params(seed=7, gridSize=(13, 9, 11), ndims=ndims, resMode=res, density_n_comp=dn, app_n_comp=an,
                            feature_init="uniform")
@@ -183,13 +183,13 @@ def _check_render(p, rays, tol, S=-1, white_bg=True, **kw):
     out, extra = _model(p, **kw)(rays, white_bg=white_bg, N_samples=S)
     assert extra == {} and set(out) == {"rgb_map", "depth_map"}
     # rays holding a sample whose weight sits within rounding of the threshold may differ by that sample
-    band = ((ref["weight"] - p.rayMarch_weight_thres).abs() < 2e-6).any(-1)
+    band = ((ref["weight"] - p.rayMarch_weight_thres).abs() < 2e-7).any(-1)
     ok = ~band
     d_rgb = (out["rgb_map"].cpu() - ref["rgb_map"]).abs().max(-1).values
     d_dep = (out["depth_map"].cpu() - ref["depth_map"]).abs()
     assert d_rgb[ok].max().item() <= tol, f"rgb max diff {d_rgb[ok].max().item()}"
     assert d_dep[ok].max().item() <= tol, f"depth max diff {d_dep[ok].max().item()}"
-    assert int(band.sum()) <= max(2, rays.shape[0] // 2000)
+    assert int(band.sum()) <= max(2, rays.shape[0] // 500)
     if band.any():
         assert d_rgb[band].max().item() <= 2e-3
     return ref, out
