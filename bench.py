@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X GridNeRF render path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c1|c2|c3|c5] ...
+
+A step is one pass of the render path over one synthetic frame (or one batch of the
+isolated-kernel workloads).  Inputs are resident in HBM before the timed region.  One
+JSON line is printed: whole-frame throughput in Mrays/s (`value`), the per-stage kernel
+times measured with HIP events inside the timed region, the roofline figure of the
+dominant kernel, and the CPU oracle timed on this box's host cores on a bounded sample
+of the same workload.
+
+Default workload: BASELINE config 4, a full 1920x1080 frame of a multi-resolution GridNeRF
+(levels 1024^2/2048^2/4096^2, 16 + 48 channels fp32, 256^3 occupancy at ~30 %, 128
+samples per ray).  The density shift is 0 so that every stage does work (with the stated
+N(0, 0.1) init and shift -10 every weight stays below the 1e-3 threshold and the colour
+network never runs; `--density-shift -10` reproduces that case).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0, "bf16": 2500.0, "f16x2": 2500.0}
+MLP_FLOP_PER_ROW = 2 * (150 * 128 + 128 * 128 + 128 * 3)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def plane_bytes_per_sample(planes):
+    return sum(4 * pl.C * (4 if pl.dtype == 0 else 2) for pl in planes)
+
+
+# ----------------------------------------------------------------------------------------
+def bench_frame(args, workload):
+    from landmark_amd import _lib as L
+    from landmark_amd import scenes
+    from landmark_amd.model import GridNeRFHIP
+
+    dev = "cuda:0"
+    t0 = time.time()
+    if workload == "c4":
+        p = scenes.c4_scene(P=args.planes, base=args.base, device=dev, density_shift=args.density_shift)
+        H, W = args.height, args.width
+        rays = scenes.c4_rays(H, W, frame=args.frame, device=dev)
+        name = f"c4_1080p_multires_P{args.planes}_base{args.base}_shift{args.density_shift:g}"
+    elif workload == "c1":
+        p = scenes.c1_scene(dense=args.density_shift == 0.0, device=dev)
+        H, W = 400, 400
+        rays = scenes.c1_rays(H, W, device=dev)
+        name = f"c1_tiny_400x400_shift{args.density_shift:g}"
+    elif workload == "c5":
+        p = scenes.c5_scene(res=args.base * 8, device=dev, density_shift=args.density_shift)
+        H, W = 2160, 3840
+        rays = scenes.c5_rays(H, W, device=dev)
+        name = f"c5_4k_cityblock_res{args.base * 8}"
+    else:
+        raise ValueError(workload)
+    model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=args.term_eps)
+    torch.cuda.synchronize()
+    log(f"[bench] scene {name} built in {time.time() - t0:.1f}s; tables "
+        f"{sum(t.numel() * t.element_size() for t in model._tables) / 1e9:.2f} GB")
+    N = rays.shape[0]
+    S = model._samples_for(-1)
+    chunk = min(args.chunk, N)
+    while chunk * S >= 2**32:
+        chunk //= 2
+    n_chunks = (N + chunk - 1) // chunk
+    rgb = torch.empty((N, 3), device=dev)
+    depth = torch.empty((N,), device=dev)
+    counters = torch.zeros((n_chunks, L.LM_STAT_WORDS), dtype=torch.int32, device=dev)
+    model.workspace(chunk, S)
+    n_ev = L.LM_N_STAGES + 1
+    events = [[[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(n_chunks)] for _ in range(args.steps)]
+    for per_step in events:
+        for per_chunk in per_step:
+            for e in per_chunk:
+                e.record()  # creates the underlying hipEvent handle
+
+    def frame(ev=None):
+        for ci in range(n_chunks):
+            sl = slice(ci * chunk, min((ci + 1) * chunk, N))
+            model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci],
+                              events=None if ev is None else ev[ci])
+
+    for _ in range(args.warmup):
+        frame()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        frame(events[k])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt / args.steps * 1e3
+
+    cnt = counters.cpu().long() & 0xFFFFFFFF
+    n_valid, n_app = int(cnt[:, L.LM_STAT_N_VALID].sum()), int(cnt[:, L.LM_STAT_N_APP].sum())
+    stage_ms = [0.0] * L.LM_N_STAGES  # per frame, averaged over steps
+    for per_step in events:
+        for per_chunk in per_step:
+            for s in range(L.LM_N_STAGES):
+                stage_ms[s] += per_chunk[s].elapsed_time(per_chunk[s + 1])
+    stage_ms = [x / args.steps for x in stage_ms]
+    launches = n_chunks  # one launch of each stage kernel per chunk
+    dens_B = plane_bytes_per_sample(model._density) + 8  # + list index in, sigma out
+    app_B = plane_bytes_per_sample(model._app) + 4 + 27 * 4  # + index in, projected features out
+    stages = {}
+    for i, nm in enumerate(L.STAGE_NAMES):
+        stages[nm] = {"ms_per_frame": round(stage_ms[i], 4)}
+    stages["density"].update(bytes_per_sample=dens_B, GBps=round(n_valid * dens_B / (stage_ms[1] * 1e-3) / 1e9, 1))
+    stages["app_gather"].update(bytes_per_sample=app_B, GBps=round(n_app * app_B / max(stage_ms[3], 1e-9) / 1e6, 1))
+    stages["colour"].update(TFLOPs=round(n_app * (MLP_FLOP_PER_ROW + 2 * model.K_app * 27) / max(stage_ms[4], 1e-9) / 1e9, 2))
+    cull_B = 32 + 0.125  # 8 corner loads of the float volume per in-box sample (upper bound: every sample), bitmap out
+    stages["cull"].update(GBps=round((N * S * cull_B + n_valid * 4) / (stage_ms[0] * 1e-3) / 1e9, 1))
+    stages["weights"].update(GBps=round((n_valid * 4 + N * S / 8 + n_app * 8 + N * 8) / (stage_ms[2] * 1e-3) / 1e9, 1))
+
+    # dominant kernel -> roofline object
+    cand = {"density": stage_ms[1], "app_gather": stage_ms[3], "colour": stage_ms[4]}
+    dom = max(cand, key=cand.get)
+    if dom == "colour":
+        ach = stages["colour"]["TFLOPs"]
+        peak = MFMA_PEAK_TFLOPS[args.mlp]
+        roof = {"kernel": "k_mlp", "bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s",
+                "frac": round(ach / peak, 4), "traffic": None}
+    else:
+        ach = stages[dom]["GBps"]
+        roof = {"kernel": "k_density_list" if dom == "density" else "k_app_feat", "bound": "hbm", "achieved": ach,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
+    roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
+    roof["launches_per_frame"] = launches
+
+    cpu, parity = cpu_baseline_frame(args, p, rays, rgb, depth, H, W)
+    mrays = N / (ms_step * 1e-3) / 1e6
+    out = {
+        "metric": "render_throughput", "value": round(mrays, 3), "unit": "Mrays/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32" if args.mlp == "f32" else f"f32+{args.mlp}-mlp",
+        "data": "synthetic",
+        "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "mlp": args.mlp,
+                   "term_eps": args.term_eps, "valid_samples": n_valid, "app_samples": n_app},
+        "frames_per_s": round(1e3 / ms_step, 3), "mpixel_per_s": round(mrays, 3),
+        "gather_GBps": stages["density"]["GBps"], "gather_frac_of_hbm_peak": round(stages["density"]["GBps"] / HBM_PEAK_GBS, 4),
+        "stages": stages, "roofline": roof, "cpu_baseline": cpu, "parity": parity,
+    }
+    return out
+
+
+def cpu_baseline_frame(args, p, rays, rgb, depth, H, W):
+    """The CPU oracle on a bounded sample of the frame (evenly spaced scan-lines)."""
+    if args.no_cpu:
+        return None, None
+    from oracle import gridnerf_oracle as O
+
+    rows = max(1, min(H, args.cpu_rows))
+    ys = torch.linspace(0, H - 1, rows).long().unique()
+    idx = (ys[:, None] * W + torch.arange(W)[None]).reshape(-1)
+    t0 = time.time()
+    pc = p.to("cpu")
+    log(f"[bench] cpu copy of the model {time.time() - t0:.1f}s")
+    r = rays[idx.to(rays.device)].cpu()
+    torch.set_num_threads(os.cpu_count() if args.cpu_threads <= 0 else args.cpu_threads)
+    t0 = time.perf_counter()
+    ret, _ = O.renderer_fn(r, pc, chunk=8192, white_bg=True)
+    dt = time.perf_counter() - t0
+    d_rgb = (rgb[idx.to(rgb.device)].cpu() - ret["rgb_map"]).abs().max().item()
+    d_dep = (depth[idx.to(rgb.device)].cpu() - ret["depth_map"]).abs().max().item()
+    cpu = {"value": round(r.shape[0] / dt / 1e6, 5), "unit": "Mrays/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"{len(ys)} evenly spaced scan-lines ({r.shape[0]} rays) of the same frame, PyTorch oracle, "
+                     f"chunk 8192, {dt:.1f}s"}
+    parity = {"rays_checked": int(r.shape[0]), "max_abs_rgb": d_rgb, "max_abs_depth": d_dep}
+    return cpu, parity
+
+
+# ----------------------------------------------------------------------------------------
+def bench_gather(args):
+    """BASELINE config 2: isolated plane/line gather, 3 planes 2048^2 x 64 ch fp32, 2^24 queries."""
+    from landmark_amd import scenes
+    from landmark_amd.model import GridNeRFHIP
+
+    dev = "cuda:0"
+    res = args.base * 2
+    p = scenes.make_params(seed=2, gridSize=(res, res, res), ndims=3, resMode=(1,), density_n_comp=64, app_n_comp=16,
+                           device=dev, feature_init="uniform")
+    model = GridNeRFHIP(p, device=dev)
+    M = args.queries
+    g = torch.Generator(device=dev).manual_seed(2)
+    xyz = torch.rand((M, 3), device=dev, generator=g) * 2 - 1
+    if args.coherent:
+        xyz = xyz[torch.argsort((xyz[:, 0] * 64).floor() * 4096 + (xyz[:, 1] * 64).floor())]
+    out = model.compute_densityfeature(xyz)
+    for _ in range(args.warmup):
+        model.compute_densityfeature(xyz)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for k in range(args.steps):
+        out = model.compute_densityfeature(xyz)
+        ev[k + 1].record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ker_ms = sum(ev[k].elapsed_time(ev[k + 1]) for k in range(args.steps)) / args.steps
+    Bq = plane_bytes_per_sample(model._density) + 12 + 4
+    gbs = M * Bq / (ker_ms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        from oracle import gridnerf_oracle as O
+
+        pc, sub = p.to("cpu"), xyz[: 1 << 20].cpu()
+        t0 = time.perf_counter()
+        ref = O.density_feature(pc, sub)
+        cdt = time.perf_counter() - t0
+        err = (out[: 1 << 20].cpu() - ref).abs().max().item()
+        cpu = {"value": round(sub.shape[0] / cdt / 1e6, 4), "unit": "Mqueries/s", "cores": torch.get_num_threads(),
+               "kind": "port", "sample": f"first 2^20 queries, F.grid_sample oracle, {cdt:.1f}s, max|diff| {err:.2e}"}
+    return {
+        "metric": "gather_throughput", "value": round(M / (dt / args.steps) / 1e6, 2), "unit": "Mqueries/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt / args.steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"c2_gather_3x{res}^2x64ch_{M}q_{'coherent' if args.coherent else 'random'}"},
+        "roofline": {"kernel": "k_density_xyz", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_ms": round(ker_ms, 4), "bytes_per_query": Bq},
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_mlp(args):
+    """BASELINE config 3: isolated colour network on 2^23 rows."""
+    from landmark_amd import scenes
+    from landmark_amd.model import GridNeRFHIP
+
+    dev = "cuda:0"
+    p = scenes.make_params(seed=3, gridSize=(8, 8, 8), density_n_comp=4, app_n_comp=48)
+    prec = args.mlp
+    model = GridNeRFHIP(p, device=dev, mlp_precision=prec)
+    M = args.rows
+    g = torch.Generator(device=dev).manual_seed(3)
+    feat = torch.randn((M, 27), device=dev, generator=g)
+    view = torch.nn.functional.normalize(torch.randn((M, 3), device=dev, generator=g), dim=-1)
+    for _ in range(args.warmup):
+        out = model.render_module(view, feat)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for k in range(args.steps):
+        out = model.render_module(view, feat)
+        ev[k + 1].record()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ker_ms = sum(ev[k].elapsed_time(ev[k + 1]) for k in range(args.steps)) / args.steps
+    tf = M * MLP_FLOP_PER_ROW / (ker_ms * 1e-3) / 1e12
+    cpu = None
+    if not args.no_cpu:
+        from oracle import gridnerf_oracle as O
+
+        n = 1 << 20
+        t0 = time.perf_counter()
+        ref = O.mlp_render(p, view[:n].cpu(), feat[:n].cpu())
+        cdt = time.perf_counter() - t0
+        err = (out[:n].cpu() - ref).abs().max().item()
+        cpu = {"value": round(n / cdt / 1e6, 4), "unit": "Mrows/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"first 2^20 rows, PyTorch oracle, {cdt:.1f}s, max|diff| {err:.2e}"}
+    return {
+        "metric": "mlp_throughput", "value": round(M / (dt / args.steps) / 1e6, 2), "unit": "Mrows/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt / args.steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": prec, "data": "synthetic",
+        "config": {"workload": f"c3_mlp_{M}rows_{prec}"},
+        "roofline": {"kernel": "k_mlp_feat", "bound": "mfma", "achieved": round(tf, 2), "peak": MFMA_PEAK_TFLOPS[prec],
+                     "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[prec], 4), "traffic": None,
+                     "avg_launch_ms": round(ker_ms, 4)},
+        "cpu_baseline": cpu,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--planes", type=int, default=3, help="ndims of the c4 model (3 = XY,XZ,YZ; 1 = XY only)")
+    ap.add_argument("--base", type=int, default=1024, help="base plane resolution of c4 (levels x1,x2,x4)")
+    ap.add_argument("--height", type=int, default=1080)
+    ap.add_argument("--width", type=int, default=1920)
+    ap.add_argument("--frame", type=int, default=0)
+    ap.add_argument("--density-shift", type=float, default=0.0)
+    ap.add_argument("--mlp", default="f16x2", choices=["f32", "f16x2", "f16", "bf16"])
+    ap.add_argument("--term-eps", type=float, default=0.0)
+    ap.add_argument("--chunk", type=int, default=65536)
+    ap.add_argument("--queries", type=int, default=1 << 24)
+    ap.add_argument("--rows", type=int, default=1 << 23)
+    ap.add_argument("--coherent", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=8)
+    ap.add_argument("--cpu-threads", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build renders on one GPU; rays are independent, so more GPUs would each take a slice of "
+              "the pixel array, but nothing here launches a second rank. Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    if args.workload == "c2":
+        out = bench_gather(args)
+    elif args.workload == "c3":
+        out = bench_mlp(args)
+    else:
+        out = bench_frame(args, args.workload)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

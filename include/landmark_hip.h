@@ -42,8 +42,11 @@ typedef enum lm_status {
 enum { LM_F32 = 0, LM_F16 = 1 };                   /* plane / line storage type */
 enum { LM_SAMPLER_AABB = 0, LM_SAMPLER_HULL = 1 }; /* sampling_opt 0 / 1 */
 enum { LM_ACT_SOFTPLUS = 0, LM_ACT_RELU = 1 };     /* fea2denseAct */
-/* arithmetic of the colour network's matrix products (accumulation is always fp32) */
-enum { LM_MLP_F32 = 0, LM_MLP_F16 = 1, LM_MLP_BF16 = 2 };
+/* arithmetic of the colour network's and basis_mat's matrix products (accumulation is
+ * always fp32).  F16X2 splits every operand into two fp16 parts (x = hi + lo) and forms
+ * hi*hi + lo*hi + hi*lo with three fp16 MFMAs: about 21 mantissa bits, for results that
+ * must stay within 1e-4 of an fp32 evaluation. */
+enum { LM_MLP_F32 = 0, LM_MLP_F16 = 1, LM_MLP_BF16 = 2, LM_MLP_F16X2 = 3 };
 
 /* One feature plane with its line (one entry of density_plane/density_line or
  * app_plane/app_line, app/models/gridnerf_sequential.py:676-718).  ax0/ax1 select the
@@ -83,6 +86,17 @@ typedef struct lm_geom {
     float vol_thre; /* alpha_mask_filter_thre */
 } lm_geom;
 
+/* stages of lm_render, in launch order */
+enum {
+    LM_STAGE_CULL = 1,      /* sampling + culling + compaction (3 kernels) */
+    LM_STAGE_DENSITY = 2,   /* density gather over the valid list */
+    LM_STAGE_WEIGHTS = 3,   /* per-ray scan, appearance list */
+    LM_STAGE_APP = 4,       /* appearance gather */
+    LM_STAGE_COLOUR = 5,    /* basis_mat + encoding + colour network */
+    LM_STAGE_COMPOSITE = 6, /* per-ray colour sum */
+    LM_N_STAGES = 6
+};
+
 typedef struct lm_model {
     lm_geom geom;
     int32_t n_planes; /* ndims * levels, plane index k = dim * levels + level */
@@ -96,6 +110,10 @@ typedef struct lm_model {
     const void *mlp_packed; /* device copy of the buffer written by lm_mlp_pack */
     int32_t white_bg;
     float term_eps; /* > 0: stop marching a ray once transmittance < term_eps */
+    /* Optional timing hooks: hipEvent_t handles created by the caller, or NULL.  lm_render
+     * records events[0] before its first kernel and events[i] after stage i on `stream`
+     * (LM_STAGE_*); it never waits on them. */
+    void *events[LM_N_STAGES + 1];
 } lm_model;
 
 /* Counters written by lm_render (device memory, 8 x uint32). */
@@ -165,26 +183,29 @@ int lm_basis(int32_t prec, const void *packed, int32_t K_basis, const float *pro
  * threshold (gridnerf_sequential.py:479/553) and the sums of :493-504 / :565-576;
  * prior art compute_beta.cuda + compute_weight.cuda (dist_render/kernel/cuda_kernel/volrend).
  *   sigma       [n_valid] densities of the valid samples, in valid-list order
- *   weight_out  optional [N*S] dense weights (NULL to skip)
- *   app_bits    [N * ceil(S/64)] uint64: bit l of word (r, c) = sample 64c+l of ray r has weight > thres
- *   app_base    [N * ceil(S/64)] uint32: slot of the first such sample of that word in app_idx
- *   app_idx     [capacity N*S] uint32 flat indices of those samples (slot order)
+ *   w_valid     [n_valid] out: their weights (same order)
+ *   weight_out  optional [N*S] dense weights; only valid samples are written (NULL to skip)
+ *   app_first   [N] uint32: slot of the ray's first sample with weight > thres in app_idx
+ *   app_cnt     [N] uint32: number of such samples; a ray's slots are contiguous and in
+ *               sample order, the order of rays in the list is not defined
+ *   app_idx     [capacity N*S] uint32 flat indices of those samples
  *   app_w       [capacity N*S] float their weights
- *   acc, depth  [N]
+ *   acc, depth  [N] sum of weights, sum of weight * z
+ *   counters    counters[LM_STAT_N_APP] is incremented by the number of listed samples
  */
 int lm_weights(const lm_geom *geom, const float *rays, int64_t N, const uint64_t *bitmap,
                const uint32_t *word_prefix, const float *sigma, float distance_scale, float weight_thres,
-               float term_eps, float *weight_out, uint64_t *app_bits, uint32_t *app_base, uint32_t *app_idx,
-               float *app_w, float *acc, float *depth, uint32_t *counters, void *stream);
+               float term_eps, float *w_valid, float *weight_out, uint32_t *app_first, uint32_t *app_cnt,
+               uint32_t *app_idx, float *app_w, float *acc, float *depth, uint32_t *counters, void *stream);
 
 /* ---- whole chunk ---------------------------------------------------------------------
  * GridBaseSequential.forward(rays_chunk, white_bg, is_train=False)
  * (gridnerf_sequential.py:439-658) -> rgb_map [N,3], depth_map [N].
- * workspace: lm_render_workspace_bytes(N, S, K_app) bytes of device memory, reusable
+ * workspace: lm_render_workspace_bytes(model, N) bytes of device memory, reusable
  * across calls (the role of MultiBlockParallelCuda.allocate_tensors,
  * dist_render/kernel/cuda_render_extend.py:35-159).  counters: [LM_STAT_WORDS] uint32
  * device memory, may be NULL.  No host synchronisation happens inside. */
-size_t lm_render_workspace_bytes(int64_t N, int32_t S, int32_t K_app);
+size_t lm_render_workspace_bytes(const lm_model *model, int64_t N);
 int lm_render(const lm_model *model, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
               float *rgb_map, float *depth_map, uint32_t *counters, void *stream);
 
@@ -193,6 +214,11 @@ int lm_density_valid(const lm_model *model, const float *rays, const uint32_t *v
                      const uint32_t *counters, float *sigma, void *stream);
 int lm_app_products(const lm_model *model, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
                     float *products, void *stream);
+/* appearance samples (list order) -> feat [n_app,27] = basis_mat(plane*line products): the
+ * gather fused with the projection, GridNeRF.compute_appfeature (gridnerf_sequential.py:829-871).
+ * Needs equal channel counts per plane, a multiple of 16 (8 with LM_MLP_F32). */
+int lm_app_features(const lm_model *model, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
+                    float *feat, void *stream);
 
 #ifdef __cplusplus
 }

@@ -12,12 +12,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(HERE, "liblandmark_hip.so")
 
 LM_MAX_PLANES = 12
+LM_N_STAGES = 6
+STAGE_NAMES = ["cull", "density", "weights", "app_gather", "colour", "composite"]
 LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_WORDS = 0, 1, 8
 LM_F32, LM_F16 = 0, 1
 LM_SAMPLER_AABB, LM_SAMPLER_HULL = 0, 1
 LM_ACT_SOFTPLUS, LM_ACT_RELU = 0, 1
-LM_MLP_F32, LM_MLP_F16, LM_MLP_BF16 = 0, 1, 2
-MLP_PREC = {"f32": LM_MLP_F32, "fp32": LM_MLP_F32, "f16": LM_MLP_F16, "fp16": LM_MLP_F16, "bf16": LM_MLP_BF16}
+LM_MLP_F32, LM_MLP_F16, LM_MLP_BF16, LM_MLP_F16X2 = 0, 1, 2, 3
+MLP_PREC = {"f32": LM_MLP_F32, "fp32": LM_MLP_F32, "f16": LM_MLP_F16, "fp16": LM_MLP_F16, "bf16": LM_MLP_BF16, "f16x2": LM_MLP_F16X2}
 
 
 class LmPlane(C.Structure):
@@ -43,6 +45,7 @@ class LmModel(C.Structure):
         ("density", LmPlane * LM_MAX_PLANES), ("app", LmPlane * LM_MAX_PLANES),
         ("act", C.c_int32), ("density_shift", C.c_float), ("distance_scale", C.c_float), ("weight_thres", C.c_float),
         ("mlp_prec", C.c_int32), ("mlp_packed", C.c_void_p), ("white_bg", C.c_int32), ("term_eps", C.c_float),
+        ("events", C.c_void_p * (LM_N_STAGES + 1)),
     ]
 
 
@@ -60,8 +63,9 @@ SYMBOLS = {
     "lm_mlp_pack": (C.c_int, [_I32, _I32, _P, _P, _P, _P, _P, _P, _P, _P]),
     "lm_mlp": (C.c_int, [_I32, _P, _I32, _P, _P, _I64, _P, _P]),
     "lm_basis": (C.c_int, [_I32, _P, _I32, _P, _I64, _P, _P]),
-    "lm_weights": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
-    "lm_render_workspace_bytes": (_SZ, [_I64, _I32, _I32]),
+    "lm_weights": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "lm_render_workspace_bytes": (_SZ, [C.POINTER(LmModel), _I64]),
+    "lm_app_features": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
     "lm_render": (C.c_int, [C.POINTER(LmModel), _P, _I64, _P, _SZ, _P, _P, _P, _P]),
     "lm_density_valid": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
     "lm_app_products": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),

@@ -74,11 +74,14 @@ extern "C" int lm_relayout_nchw_to_hwc(const void *src, void *dst, int32_t C, in
 // ---- whole chunk -------------------------------------------------------------------------------
 int lm_check_geom(const lm_geom *g);
 int lm_check_planes(const lm_plane *planes, int32_t n, int *dtype_out, int *K_out);
-int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *products, const float *rays,
+int lm_app_feat_supported(const lm_model *m);
+int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *feat, const float *rays,
                          const uint32_t *app_idx, const uint32_t *count, float *rgb, hipStream_t stream);
-int lm_launch_composite(int64_t N, int S, const uint64_t *app_bits, const uint32_t *app_base, const float *app_w,
+int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
                         const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream);
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
+int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
+                    float *feat, hipStream_t st);
 
 namespace {
 struct Workspace {
@@ -87,18 +90,20 @@ struct Workspace {
     void *cull_scratch;
     uint32_t *valid_idx;
     float *sigma;
-    uint64_t *app_bits;
-    uint32_t *app_base;
+    float *w_valid;
+    uint32_t *app_first;
+    uint32_t *app_cnt;
     uint32_t *app_idx;
     float *app_w;
     float *rgb;
-    float *products;
+    float *feat;
+    float *products;  // only when the fused appearance gather does not cover the model
     float *acc;
     uint32_t *counters;
     size_t total;
 };
 
-Workspace carve(char *base, int64_t N, int32_t S, int32_t K) {
+Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products) {
     Workspace w;
     size_t o = 0;
     auto take = [&](size_t bytes) {
@@ -106,62 +111,88 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K) {
         o = (o + bytes + 255) & ~(size_t)255;
         return p;
     };
-    const uint64_t total = (uint64_t)N * (uint64_t)S, n_words = (total + 63) / 64, steps = (uint64_t)(S + 63) / 64;
-    // a ray's weights sum to at most 1, so at most min(S, 1/threshold) of them can exceed the
-    // threshold; without knowing the threshold the capacity is N*S
+    const uint64_t total = (uint64_t)N * (uint64_t)S, n_words = (total + 63) / 64;
+    // every sample may be valid and (for S below 1/threshold) above the weight threshold
     const uint64_t cap = total;
     w.bitmap = (uint64_t *)take(n_words * 8);
     w.word_prefix = (uint32_t *)take(n_words * 4);
     w.cull_scratch = take(lm_sample_cull_scratch_bytes(N, S));
     w.valid_idx = (uint32_t *)take(total * 4);
     w.sigma = (float *)take(total * 4);
-    w.app_bits = (uint64_t *)take((uint64_t)N * steps * 8);
-    w.app_base = (uint32_t *)take((uint64_t)N * steps * 4);
+    w.w_valid = (float *)take(total * 4);
+    w.app_first = (uint32_t *)take((uint64_t)N * 4);
+    w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
     w.app_idx = (uint32_t *)take(cap * 4);
     w.app_w = (float *)take(cap * 4);
     w.rgb = (float *)take(cap * 12);
-    w.products = (float *)take(cap * (uint64_t)K * 4);
+    w.feat = (float *)take(cap * 27 * 4);
+    w.products = need_products ? (float *)take(cap * (uint64_t)K * 4) : nullptr;
     w.acc = (float *)take((uint64_t)N * 4);
     w.counters = (uint32_t *)take(LM_STAT_WORDS * 4);
     w.total = o;
     return w;
 }
+
+int check_model(const lm_model *m, int *K) {
+    LM_REQUIRE(m != nullptr, "model is null");
+    if (int rc = lm_check_geom(&m->geom)) return rc;
+    int dt;
+    if (int rc = lm_check_planes(m->density, m->n_planes, &dt, nullptr)) return rc;
+    if (int rc = lm_check_planes(m->app, m->n_planes, &dt, K)) return rc;
+    return LM_OK;
+}
 }  // namespace
 
-extern "C" size_t lm_render_workspace_bytes(int64_t N, int32_t S, int32_t K_app) {
-    if (N <= 0 || S <= 0 || K_app <= 0) return 0;
-    return carve(nullptr, N, S, K_app).total;
+extern "C" size_t lm_render_workspace_bytes(const lm_model *m, int64_t N) {
+    int K;
+    if (check_model(m, &K) || N <= 0) return 0;
+    return carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m)).total;
 }
 
 extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
                          float *rgb_map, float *depth_map, uint32_t *counters, void *stream) {
-    LM_REQUIRE(m != nullptr, "model is null");
-    if (int rc = lm_check_geom(&m->geom)) return rc;
-    int dt, K;
-    if (int rc = lm_check_planes(m->density, m->n_planes, &dt, nullptr)) return rc;
-    if (int rc = lm_check_planes(m->app, m->n_planes, &dt, &K)) return rc;
+    int K;
+    if (int rc = check_model(m, &K)) return rc;
     LM_REQUIRE(N >= 0, "negative ray count");
     if (N == 0) return LM_OK;
     LM_REQUIRE(rays && rgb_map && depth_map, "null buffer");
     LM_REQUIRE(workspace && lm_aligned16(workspace), "workspace is null or misaligned");
     const int S = m->geom.S;
     LM_REQUIRE((uint64_t)N * (uint64_t)S < (1ull << 32), "N*S does not fit 32-bit sample indices; split the chunk");
-    Workspace w = carve((char *)workspace, N, S, K);
+    const bool fused = lm_app_feat_supported(m) != 0;
+    Workspace w = carve((char *)workspace, N, S, K, !fused);
     if (w.total > workspace_bytes)
         LM_FAIL(LM_ERR_WORKSPACE, "workspace has %zu bytes, %zu needed for N=%lld S=%d K=%d", workspace_bytes, w.total,
                 (long long)N, S, K);
     hipStream_t st = (hipStream_t)stream;
     uint32_t *cnt = counters ? counters : w.counters;
+    auto mark = [&](int i) {
+        if (m->events[i]) (void)hipEventRecord((hipEvent_t)m->events[i], st);
+    };
+    mark(0);
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
     if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, w.valid_idx, cnt, nullptr, w.cull_scratch, st))
         return rc;
+    mark(LM_STAGE_CULL);
     if (int rc = lm_density_valid(m, rays, w.valid_idx, cnt, w.sigma, st)) return rc;
+    mark(LM_STAGE_DENSITY);
     if (int rc = lm_weights(&m->geom, rays, N, w.bitmap, w.word_prefix, w.sigma, m->distance_scale, m->weight_thres,
-                            m->term_eps, nullptr, w.app_bits, w.app_base, w.app_idx, w.app_w, w.acc, depth_map, cnt, st))
+                            m->term_eps, w.w_valid, nullptr, w.app_first, w.app_cnt, w.app_idx, w.app_w, w.acc, depth_map,
+                            cnt, st))
         return rc;
-    if (int rc = lm_app_products(m, rays, w.app_idx, cnt, w.products, st)) return rc;
-    if (int rc = lm_launch_app_colour(m->mlp_prec, m->mlp_packed, K, S, w.products, rays, w.app_idx,
-                                      cnt + LM_STAT_N_APP, w.rgb, st))
+    mark(LM_STAGE_WEIGHTS);
+    if (fused) {
+        if (int rc = lm_app_features(m, rays, w.app_idx, cnt, w.feat, st)) return rc;
+    } else {
+        // channel counts the fused kernel does not cover: products through memory, then basis_mat
+        if (int rc = lm_app_products(m, rays, w.app_idx, cnt, w.products, st)) return rc;
+        if (int rc = lm_launch_basis(m->mlp_prec, m->mlp_packed, K, w.products, 0, cnt + LM_STAT_N_APP, w.feat, st)) return rc;
+    }
+    mark(LM_STAGE_APP);
+    if (int rc = lm_launch_app_colour(m->mlp_prec, m->mlp_packed, K, S, w.feat, rays, w.app_idx, cnt + LM_STAT_N_APP, w.rgb, st))
         return rc;
-    return lm_launch_composite(N, S, w.app_bits, w.app_base, w.app_w, w.rgb, w.acc, m->white_bg, rgb_map, st);
+    mark(LM_STAGE_COLOUR);
+    if (int rc = lm_launch_composite(N, w.app_first, w.app_cnt, w.app_w, w.rgb, w.acc, m->white_bg, rgb_map, st)) return rc;
+    mark(LM_STAGE_COMPOSITE);
+    return LM_OK;
 }

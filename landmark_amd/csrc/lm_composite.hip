@@ -1,13 +1,15 @@
-// Part 4: volume compositing as a per-ray segmented scan.
+// Part 4: volume compositing as a per-ray segmented scan over the valid samples only.
 //
-// k_weights: one wave per ray, 64 samples per step.  Each lane recomputes its sample's
-// depth with the sampler's own operations, fetches sigma through the bitmap / word-prefix
-// (invalid samples have sigma = 0, exactly like the reference's zero-initialised tensor),
-// forms alpha, and a multiplicative wave scan yields the transmittance.  Samples whose
-// weight exceeds the threshold are appended to the appearance list: one atomic per wave
-// step reserves a contiguous slot range, and the (base, bit mask) pair is kept per ray so
-// that the final sum runs over a ray's samples in sample order whatever the slot order was.
-// k_composite: one thread per ray sums weight * rgb over those slots, adds the white
+// k_weights: one lane per ray.  The ray's valid samples are the set bits of its slice of
+// the sample bitmap; their densities sit contiguously in the compacted sigma array.  The
+// lane walks those bits in sample order and carries the transmittance along, which is
+// exactly the sequential product torch.cumprod forms; culled samples have sigma = 0 in the
+// reference, i.e. alpha = 0 and a factor (1 - 0 + 1e-10) that rounds to 1.0f, so skipping
+// them changes nothing.  Two passes: the first stores the weights of the valid samples and
+// counts those above the threshold, a wave-wide prefix sum plus one atomic per wave reserves
+// a contiguous slot range per ray in the appearance list, the second pass fills the slots.
+// A ray's slots are therefore contiguous and in sample order.
+// k_composite: one lane per ray sums weight * rgb over its slots, adds the white
 // background and clamps.
 //
 // Reference: raw2alpha (app/tools/utils.py:51-64), dists with a zero last interval
@@ -18,111 +20,136 @@
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kRaysPerBlock = kBlock / LM_WAVE;
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
-    return v;
-}
+struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
+    const uint64_t *bitmap;
+    const uint32_t *prefix;
+    uint64_t w, w_last, bits, flat1;
+    uint32_t pos;
+    __device__ __forceinline__ void start(const uint64_t *bm, const uint32_t *pf, uint64_t flat0, uint64_t flat1_) {
+        bitmap = bm; prefix = pf; flat1 = flat1_;
+        w = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
+        const uint64_t raw = bm[w];
+        const unsigned b0 = (unsigned)(flat0 & 63);
+        const uint64_t below = b0 ? ((1ull << b0) - 1ull) : 0ull;
+        pos = pf[w] + (uint32_t)__popcll(raw & below);
+        bits = mask_tail(raw & ~below);
+    }
+    __device__ __forceinline__ uint64_t mask_tail(uint64_t x) const {
+        if (w == w_last) {
+            const unsigned e = (unsigned)(flat1 & 63);
+            if (e) x &= (1ull << e) - 1ull;
+        }
+        return x;
+    }
+    // next set bit -> flat index; false when exhausted.  `pos` is the compact position of it.
+    __device__ __forceinline__ bool next(uint64_t &flat) {
+        while (bits == 0) {
+            if (w == w_last) return false;
+            ++w;
+            bits = mask_tail(bitmap[w]);
+        }
+        const int b = __ffsll((unsigned long long)bits) - 1;
+        bits &= bits - 1;
+        flat = w * 64 + (uint64_t)b;
+        return true;
+    }
+};
 
 __global__ __launch_bounds__(kBlock) void k_weights(lm_geom g, const float *__restrict__ rays, uint64_t N,
                                                     const uint64_t *__restrict__ bitmap,
                                                     const uint32_t *__restrict__ word_prefix,
                                                     const float *__restrict__ sigma, float distance_scale,
-                                                    float weight_thres, float term_eps, float *__restrict__ weight_out,
-                                                    uint64_t *__restrict__ app_bits, uint32_t *__restrict__ app_base,
-                                                    uint32_t *__restrict__ app_idx, float *__restrict__ app_w,
-                                                    float *__restrict__ acc_out, float *__restrict__ depth_out,
-                                                    uint32_t *__restrict__ app_count) {
+                                                    float weight_thres, float term_eps, float *__restrict__ w_valid,
+                                                    float *__restrict__ weight_out, uint32_t *__restrict__ app_first,
+                                                    uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ app_idx,
+                                                    float *__restrict__ app_w, float *__restrict__ acc_out,
+                                                    float *__restrict__ depth_out, uint32_t *__restrict__ app_count) {
     const unsigned lane = lm_lane();
-    const uint64_t r = (uint64_t)blockIdx.x * kRaysPerBlock + threadIdx.x / LM_WAVE;
-    if (r >= N) return;
+    const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const bool active = r < N;
     const int S = g.S;
-    const int n_steps = (S + 63) / 64;
-    float ray[6];
+    float acc = 0.0f, depth = 0.0f;
+    uint32_t cnt = 0, p_first = 0, p_end = 0;
+    float rp = 0.0f;
+    const uint64_t flat0 = r * (uint64_t)S;
+    if (active) {
+        float ray[6];
 #pragma unroll
-    for (int k = 0; k < 6; ++k) ray[k] = rays[6 * r + k];
-    const float rp = lm_ray_param(g, ray);
-    float T = 1.0f, acc = 0.0f, depth = 0.0f;
-    int step = 0;
-    for (; step < n_steps; ++step) {
-        const int s = step * 64 + (int)lane;
-        const bool in = s < S;
-        float z = 0.0f, sg = 0.0f, dist = 0.0f;
-        if (in) {
-            z = lm_sample_z(g, rp, s);
-            if (s + 1 < S) dist = lm_sample_z(g, rp, s + 1) - z;
-            const uint64_t flat = r * (uint64_t)S + s;
-            const uint64_t w = flat >> 6;
-            const unsigned b = (unsigned)(flat & 63);
-            const uint64_t bits = bitmap[w];
-            if ((bits >> b) & 1ull) sg = sigma[word_prefix[w] + (uint32_t)__popcll(bits & ((1ull << b) - 1ull))];
+        for (int k = 0; k < 6; ++k) ray[k] = rays[6 * r + k];
+        rp = lm_ray_param(g, ray);
+        BitWalk it;
+        it.start(bitmap, word_prefix, flat0, flat0 + S);
+        p_first = it.pos;
+        uint32_t p = p_first;
+        float T = 1.0f;
+        uint64_t flat;
+        while (it.next(flat)) {
+            const int s = (int)(flat - flat0);
+            const float z = lm_sample_z(g, rp, s);
+            const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
+            const float d2 = dist * distance_scale;
+            const float alpha = 1.0f - expf(-sigma[p] * d2);
+            const float wgt = alpha * T;
+            T = T * ((1.0f - alpha) + 1e-10f);
+            w_valid[p] = wgt;
+            if (weight_out) weight_out[flat] = wgt;
+            acc += wgt;
+            depth += wgt * z;
+            cnt += wgt > weight_thres;
+            ++p;
+            if (term_eps > 0.0f && T < term_eps) break;
         }
-        const float d2 = dist * distance_scale;
-        const float alpha = 1.0f - expf(-sg * d2);
-        const float x = in ? (1.0f - alpha) + 1e-10f : 1.0f;
-        float incl = x;  // inclusive product scan over the wave
+        p_end = p;
+    }
+    // slot range per ray: exclusive prefix over the wave + one atomic
+    uint32_t incl = cnt;
 #pragma unroll
-        for (int d = 1; d < LM_WAVE; d <<= 1) {
-            const float y = __shfl_up(incl, d);
-            if (lane >= (unsigned)d) incl *= y;
-        }
-        float excl = __shfl_up(incl, 1);
-        if (lane == 0) excl = 1.0f;
-        const float wgt = alpha * (T * excl);
-        T = T * __shfl(incl, LM_WAVE - 1);
-        if (in && weight_out) weight_out[r * (uint64_t)S + s] = wgt;
-        acc += wgt;
-        depth += wgt * z;
-        const bool is_app = in && (wgt > weight_thres);
-        const uint64_t abits = __ballot(is_app);
-        uint32_t base = 0;
-        if (abits) {
-            if (lane == 0) base = atomicAdd(app_count, (uint32_t)__popcll(abits));
-            base = __shfl(base, 0);
-            if (is_app) {
-                const uint32_t slot = base + lm_mbcnt(abits);
-                app_idx[slot] = (uint32_t)(r * (uint64_t)S + s);
+    for (int d = 1; d < LM_WAVE; d <<= 1) {
+        const uint32_t y = __shfl_up(incl, d);
+        if (lane >= (unsigned)d) incl += y;
+    }
+    const uint32_t total = __shfl(incl, LM_WAVE - 1);
+    uint32_t base = 0;
+    if (total) {
+        if (lane == 0) base = atomicAdd(app_count, total);
+        base = __shfl(base, 0);
+    }
+    if (!active) return;
+    uint32_t slot = base + incl - cnt;
+    app_first[r] = slot;
+    app_cnt[r] = cnt;
+    acc_out[r] = acc;
+    depth_out[r] = depth;
+    if (cnt) {
+        BitWalk it;
+        it.start(bitmap, word_prefix, flat0, flat0 + S);
+        uint64_t flat;
+        for (uint32_t p = p_first; p < p_end; ++p) {
+            it.next(flat);
+            const float wgt = w_valid[p];
+            if (wgt > weight_thres) {
+                app_idx[slot] = (uint32_t)flat;
                 app_w[slot] = wgt;
+                ++slot;
             }
         }
-        if (lane == 0) {
-            app_bits[r * n_steps + step] = abits;
-            app_base[r * n_steps + step] = base;
-        }
-        if (term_eps > 0.0f && T < term_eps) { ++step; break; }
     }
-    // steps skipped by early termination hold no appearance samples
-    for (; step < n_steps; ++step) {
-        if (lane == 0) { app_bits[r * n_steps + step] = 0; app_base[r * n_steps + step] = 0; }
-        if (weight_out) {
-            const int s = step * 64 + (int)lane;
-            if (s < S) weight_out[r * (uint64_t)S + s] = 0.0f;
-        }
-    }
-    acc = wave_sum(acc);
-    depth = wave_sum(depth);
-    if (lane == 0) { acc_out[r] = acc; depth_out[r] = depth; }
 }
 
-__global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, int n_steps, const uint64_t *__restrict__ app_bits,
-                                                      const uint32_t *__restrict__ app_base,
+__global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t *__restrict__ app_first,
+                                                      const uint32_t *__restrict__ app_cnt,
                                                       const float *__restrict__ app_w, const float *__restrict__ rgb,
                                                       const float *__restrict__ acc, int white_bg,
                                                       float *__restrict__ rgb_map) {
     const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (r >= N) return;
     float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f;
-    for (int step = 0; step < n_steps; ++step) {
-        const uint64_t bits = app_bits[r * n_steps + step];
-        const int n = __popcll(bits);
-        const uint32_t base = app_base[r * n_steps + step];
-        for (int i = 0; i < n; ++i) {
-            const float w = app_w[base + i];
-            const float *c = rgb + 3 * (size_t)(base + i);
-            c0 = fmaf(w, c[0], c0); c1 = fmaf(w, c[1], c1); c2 = fmaf(w, c[2], c2);
-        }
+    const uint32_t first = app_first[r], n = app_cnt[r];
+    for (uint32_t i = 0; i < n; ++i) {
+        const float w = app_w[first + i];
+        const float *c = rgb + 3 * (size_t)(first + i);
+        c0 = fmaf(w, c[0], c0); c1 = fmaf(w, c[1], c1); c2 = fmaf(w, c[2], c2);
     }
     if (white_bg) {
         const float bgd = 1.0f - acc[r];
@@ -143,28 +170,28 @@ int lm_check_geom(const lm_geom *g);
 
 extern "C" int lm_weights(const lm_geom *geom, const float *rays, int64_t N, const uint64_t *bitmap,
                           const uint32_t *word_prefix, const float *sigma, float distance_scale, float weight_thres,
-                          float term_eps, float *weight_out, uint64_t *app_bits, uint32_t *app_base, uint32_t *app_idx,
-                          float *app_w, float *acc, float *depth, uint32_t *counters, void *stream) {
+                          float term_eps, float *w_valid, float *weight_out, uint32_t *app_first, uint32_t *app_cnt,
+                          uint32_t *app_idx, float *app_w, float *acc, float *depth, uint32_t *counters, void *stream) {
     if (int rc = lm_check_geom(geom)) return rc;
     LM_REQUIRE(N >= 0, "negative ray count");
     LM_REQUIRE(counters != nullptr, "counters is null");
     if (N == 0) return LM_OK;
-    LM_REQUIRE(rays && bitmap && word_prefix && sigma && app_bits && app_base && app_idx && app_w && acc && depth,
+    LM_REQUIRE(rays && bitmap && word_prefix && sigma && w_valid && app_first && app_cnt && app_idx && app_w && acc && depth,
                "null buffer");
-    const unsigned grid = (unsigned)(((uint64_t)N + kRaysPerBlock - 1) / kRaysPerBlock);
+    const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(k_weights, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, *geom, rays, (uint64_t)N, bitmap,
-                       word_prefix, sigma, distance_scale, weight_thres, term_eps, weight_out, app_bits, app_base, app_idx,
-                       app_w, acc, depth, counters + LM_STAT_N_APP);
+                       word_prefix, sigma, distance_scale, weight_thres, term_eps, w_valid, weight_out, app_first, app_cnt,
+                       app_idx, app_w, acc, depth, counters + LM_STAT_N_APP);
     LM_CHECK_LAUNCH("k_weights");
     return LM_OK;
 }
 
-int lm_launch_composite(int64_t N, int S, const uint64_t *app_bits, const uint32_t *app_base, const float *app_w,
+int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
                         const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream) {
     if (N == 0) return LM_OK;
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(k_composite, dim3(grid), dim3(kBlock), 0, stream, (uint64_t)N, (S + 63) / 64, app_bits, app_base,
-                       app_w, rgb, acc, white_bg, rgb_map);
+    hipLaunchKernelGGL(k_composite, dim3(grid), dim3(kBlock), 0, stream, (uint64_t)N, app_first, app_cnt, app_w, rgb, acc,
+                       white_bg, rgb_map);
     LM_CHECK_LAUNCH("k_composite");
     return LM_OK;
 }

@@ -13,6 +13,7 @@
 #include <hip/hip_fp16.h>
 
 #include "lm_common.h"
+#include "lm_mma.h"
 
 namespace {
 
@@ -242,6 +243,150 @@ __global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int
     }
 }
 
+
+// ---- appearance gather fused with basis_mat --------------------------------------------------
+// One wave owns 32 appearance samples; lane (j, h) gathers, for sample j, CW consecutive
+// channels of every group of 2*CW (the lane pair of a sample covers the group), multiplies
+// plane by line and feeds the products straight into the matrix cores as the B operand of
+// basis_mat (A = the packed basis fragments, resident in LDS).  The [n, P*L*C] product
+// matrix never exists in memory; the kernel writes the 27 projected features per sample.
+template <typename T, int CW> struct ChLoad;
+template <int CW> struct ChLoad<float, CW> {
+    __device__ static __forceinline__ void load(const float *p, float *o) {
+#pragma unroll
+        for (int i = 0; i < CW; i += 4) {
+            float4 v = *reinterpret_cast<const float4 *>(p + i);
+            o[i] = v.x; o[i + 1] = v.y; o[i + 2] = v.z; o[i + 3] = v.w;
+        }
+    }
+};
+template <> struct ChLoad<__half, 8> {
+    __device__ static __forceinline__ void load(const __half *p, float *o) { Vec<__half>::load(p, o); }
+};
+template <> struct ChLoad<__half, 4> {
+    __device__ static __forceinline__ void load(const __half *p, float *o) {
+        uint2 raw = *reinterpret_cast<const uint2 *>(p);
+        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+        float2 a = __half22float2(h[0]), b = __half22float2(h[1]);
+        o[0] = a.x; o[1] = a.y; o[2] = b.x; o[3] = b.y;
+    }
+};
+
+template <int PREC, typename T, int NU>  // NU = groups of 2*CW channels per plane
+__global__ __launch_bounds__(256) void k_app_feat(lm_geom g, PlaneSet ps, int K, const char *__restrict__ packed,
+                                                  lm_mma::PackLayout L, const float *__restrict__ rays,
+                                                  const uint32_t *__restrict__ list,
+                                                  const uint32_t *__restrict__ count, float *__restrict__ feat) {
+    using namespace lm_mma;
+    using Mm = Mma<PREC>;
+    using frag = typename Mm::frag;
+    constexpr int G = Mm::G, CW = Mm::CW, NP = Mm::NP;
+    extern __shared__ __align__(16) char lds[];
+    {
+        const size_t bytes = (size_t)32 * K * sizeof(typename Mm::elem) * NP;
+        const uint4 *src = reinterpret_cast<const uint4 *>(packed + L.basis);
+        uint4 *dst = reinterpret_cast<uint4 *>(lds);
+        for (size_t i = threadIdx.x; i < bytes / 16; i += blockDim.x) dst[i] = src[i];
+        __syncthreads();
+    }
+    const frag *A = reinterpret_cast<const frag *>(lds);
+    const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
+    const uint64_t M = *count;
+    const uint64_t n_tiles = (M + 31) / 32;
+    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * 4 + threadIdx.x / LM_WAVE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * 4;
+    for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
+        const uint64_t p = tile * 32 + j;
+        const bool live = p < M;
+        float q[3];
+        list_coords(g, rays, list[live ? p : M - 1], q);
+        floatx16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+        int t = 0;  // running MFMA step = slot / G over the concatenated channels
+        for (int k = 0; k < ps.n; ++k) {
+            const lm_plane &pl = ps.p[k];
+            const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+            const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+            const T *P = reinterpret_cast<const T *>(pl.plane);
+            const T *Ln = reinterpret_cast<const T *>(pl.line);
+            float a[NU][CW], b[NU][CW], c[NU][CW], d[NU][CW], l0[NU][CW], l1[NU][CW];
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                const int ch = 2 * CW * u + CW * (int)h;
+                ChLoad<T, CW>::load(P + t2.o00 + ch, a[u]);
+                ChLoad<T, CW>::load(P + t2.o01 + ch, b[u]);
+                ChLoad<T, CW>::load(P + t2.o10 + ch, c[u]);
+                ChLoad<T, CW>::load(P + t2.o11 + ch, d[u]);
+                ChLoad<T, CW>::load(Ln + t1.o0 + ch, l0[u]);
+                ChLoad<T, CW>::load(Ln + t1.o1 + ch, l1[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < NU; ++u) {
+                float prod[CW];
+#pragma unroll
+                for (int i = 0; i < CW; ++i) {
+                    float pv = a[u][i] * t2.w00;
+                    pv = fmaf(b[u][i], t2.w01, pv);
+                    pv = fmaf(c[u][i], t2.w10, pv);
+                    pv = fmaf(d[u][i], t2.w11, pv);
+                    const float lv = fmaf(l1[u][i], t1.w1, l0[u][i] * t1.w0);
+                    prod[i] = pv * lv;
+                }
+#pragma unroll
+                for (int s = 0; s < CW / G; ++s, ++t) {
+                    frag bf[NP];
+                    Mm::pack(prod + s * G, bf);
+                    const frag a0 = A[(t * NP) * 64 + lane];
+                    acc = Mm::mma(a0, bf[0], acc);
+                    if constexpr (NP == 2) {
+                        const frag a1 = A[(t * NP + 1) * 64 + lane];
+                        acc = Mm::mma(a1, bf[0], acc);
+                        acc = Mm::mma(a0, bf[1], acc);
+                    }
+                }
+            }
+        }
+        if (live) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = row_of(v, (int)h);
+                if (r < kAppDim) feat[p * kAppDim + r] = acc[v];
+            }
+        }
+    }
+}
+
+template <int PREC, typename T>
+int launch_app_feat(int nu, const lm_model *m, const PlaneSet &ps, int K, const float *rays, const uint32_t *list,
+                    const uint32_t *count, float *feat, hipStream_t st) {
+    using namespace lm_mma;
+    const PackLayout L = pack_layout(PREC, K);
+    const size_t lds = (size_t)32 * K * sizeof(typename Mma<PREC>::elem) * Mma<PREC>::NP;
+    if (lds > 150 * 1024) LM_FAIL(LM_ERR_UNSUPPORTED, "basis_mat fragments (%zu bytes) do not fit LDS", lds);
+    const unsigned grid = (unsigned)lm_persistent_blocks(lds > 72 * 1024 ? 1 : 2);
+#define LM_AF_CASE(NU_)                                                                                            \
+    case NU_: {                                                                                                    \
+        auto kern = &k_app_feat<PREC, T, NU_>;                                                                     \
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                  \
+        if (e != hipSuccess) LM_FAIL(LM_ERR_LAUNCH, "k_app_feat: LDS reservation failed: %s", hipGetErrorString(e)); \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, m->geom, ps, K, (const char *)m->mlp_packed, L, rays, \
+                           list, count, feat);                                                                     \
+        break;                                                                                                     \
+    }
+    switch (nu) {
+        LM_AF_CASE(1)
+        LM_AF_CASE(2)
+        LM_AF_CASE(3)
+        LM_AF_CASE(4)
+        default: LM_FAIL(LM_ERR_UNSUPPORTED, "unsupported channel grouping %d", nu);
+    }
+#undef LM_AF_CASE
+    LM_CHECK_LAUNCH("k_app_feat");
+    return LM_OK;
+}
+
 }  // namespace
 
 // -------------------------------------------------------------------------------------------
@@ -348,4 +493,49 @@ extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint3
                            app_idx, counters + LM_STAT_N_APP, products);
     LM_CHECK_LAUNCH("k_app_list");
     return LM_OK;
+}
+
+// True when the fused gather + basis_mat kernel covers this model's appearance planes.
+int lm_app_feat_supported(const lm_model *m) {
+    const int cw = m->mlp_prec == LM_MLP_F32 ? 4 : 8;
+    const int C = m->app[0].C;
+    for (int k = 0; k < m->n_planes; ++k)
+        if (m->app[k].C != C) return 0;
+    if (C % (2 * cw) != 0) return 0;
+    const int nu = C / (2 * cw);
+    return nu >= 1 && nu <= 4;
+}
+
+int lm_check_prec(int prec);
+int lm_check_K(int K);
+
+// appearance samples (list order) -> feat [n_app, 27] = basis_mat(plane * line products)
+extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
+                               float *feat, void *stream) {
+    LM_REQUIRE(m != nullptr, "model is null");
+    if (int rc = lm_check_geom(&m->geom)) return rc;
+    int dtype, K;
+    if (int rc = lm_check_planes(m->app, m->n_planes, &dtype, &K)) return rc;
+    if (int rc = lm_check_prec(m->mlp_prec)) return rc;
+    if (int rc = lm_check_K(K)) return rc;
+    LM_REQUIRE(rays && app_idx && counters && feat, "null buffer");
+    LM_REQUIRE(m->mlp_packed && lm_aligned16(m->mlp_packed), "packed colour-network weights are null or misaligned");
+    if (!lm_app_feat_supported(m))
+        LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs equal channel counts, a multiple of %d",
+                m->mlp_prec == LM_MLP_F32 ? 8 : 16);
+    const PlaneSet ps = make_set(m->app, m->n_planes);
+    const int cw = m->mlp_prec == LM_MLP_F32 ? 4 : 8;
+    const int nu = m->app[0].C / (2 * cw);
+    hipStream_t st = (hipStream_t)stream;
+    const uint32_t *cnt = counters + LM_STAT_N_APP;
+#define LM_AF_GO(PREC_)                                                                                    \
+    return dtype == LM_F32 ? launch_app_feat<PREC_, float>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
+                           : launch_app_feat<PREC_, __half>(nu, m, ps, K, rays, app_idx, cnt, feat, st)
+    switch (m->mlp_prec) {
+        case LM_MLP_F32: LM_AF_GO(LM_MLP_F32);
+        case LM_MLP_F16: LM_AF_GO(LM_MLP_F16);
+        case LM_MLP_BF16: LM_AF_GO(LM_MLP_BF16);
+        default: LM_AF_GO(LM_MLP_F16X2);
+    }
+#undef LM_AF_GO
 }

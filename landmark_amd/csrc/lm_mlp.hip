@@ -1,112 +1,49 @@
-// Part 3: appearance projection (basis_mat) + positional encoding + colour network on the
+// Part 3: positional encoding + colour network (and the basis_mat projection) on the
 // matrix cores.
 //
 // One wave owns 32 samples.  All products are computed "transposed": the weight matrix
 // is the A operand (32 output rows per MFMA), the 32 samples are the columns, so the
 // 32x32 accumulator of one layer already has the register layout the next layer needs as
 // its B operand (lane = sample, registers = features).  Activations therefore never leave
-// the register file between basis_mat, the encoding and the three layers.  The order of
-// the K dimension is free in a dot product, so the host packs every weight matrix into
-// the exact per-lane fragment order the kernel consumes (lm_mlp_pack); a wave reads one
-// contiguous fragment per MFMA.
+// the register file between the encoding and the three layers.  The order of the K
+// dimension is free in a dot product, so the host packs every weight matrix into the exact
+// per-lane fragment order the kernel consumes (lm_mlp_pack); layers 1 and 2 are copied to
+// LDS once per workgroup and every MFMA reads one contiguous, conflict-free fragment.
+//
+// Arithmetic modes (accumulation is always fp32):
+//   F32    v_mfma_f32_32x32x2_f32
+//   F16    v_mfma_f32_32x32x16_f16,  BF16  v_mfma_f32_32x32x16_bf16
+//   F16X2  every operand x is split into fp16 parts x = hi + lo; a*b is evaluated as
+//          hi*hi + lo*hi + hi*lo with three fp16 MFMAs (products of fp16 numbers are exact
+//          in fp32), which keeps ~21 mantissa bits at a quarter of the fp32 MFMA cost.
 //
 // Register layout of a 32x32 fp32 accumulator (all 32x32 MFMA shapes): lane l holds column
 // j = l%32; with h = l/32 its register v (0..15) is row 8*(v/4) + 4*h + v%4.
 //
-// Row assignment after basis_mat: rows 0..26 are the 27 appearance features, rows 28..30
-// are overwritten with the view direction, rows 27 and 31 are zero.  Each lane thus owns
-// 16 raw values (15 real); the network input is built per lane as five groups of 16:
-// raw, sin(raw), cos(raw), sin(2 raw), cos(2 raw) = 80 slots, 160 per sample (150 real,
-// the rest meet zero weights).  Reference input order it is mapped to:
-// app/models/mlp_render_fea.py:55-65 with app/tools/utils.py:42-48.
+// Row assignment of the network input: rows 0..26 are the 27 appearance features, rows
+// 28..30 the view direction, rows 27 and 31 are zero.  Each lane thus owns 16 raw values
+// (15 real); the input is built per lane as five groups of 16: raw, sin(raw), cos(raw),
+// sin(2 raw), cos(2 raw) = 80 slots, 160 per sample (150 real, the rest meet zero
+// weights).  Reference input order it is mapped to: app/models/mlp_render_fea.py:55-65
+// with app/tools/utils.py:42-48.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
-#include <vector>
 
 #include "lm_common.h"
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+#include "lm_mma.h"
 
 namespace {
 
-constexpr int kAppDim = 27;
-constexpr int kHidden = 128;
-constexpr int kInDim = 150;
-constexpr int kSlots1 = 80;  // per lane-half
-constexpr int kBlock = 256;
+using namespace lm_mma;
 
-__host__ __device__ constexpr int row_of(int v, int h) { return 8 * (v / 4) + 4 * h + (v % 4); }
+// 16-bit modes: 8 waves per workgroup (two per SIMD, 256 registers each); the split and fp32
+// modes need the full register file of a SIMD per wave
+template <int PREC> struct MlpBlock { static constexpr int N = (PREC == LM_MLP_F16 || PREC == LM_MLP_BF16) ? 512 : 256; };
 
-template <int PREC> struct Mma;
-template <> struct Mma<LM_MLP_F32> {
-    static constexpr int G = 1;   // K slots one lane feeds per MFMA
-    static constexpr int CW = 4;  // consecutive product channels a lane reads at once
-    using elem = float;
-    using frag = float;
-    __device__ static __forceinline__ floatx16 mma(frag a, frag b, floatx16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ frag pack(const float *s) { return s[0]; }
-};
-template <> struct Mma<LM_MLP_F16> {
-    static constexpr int G = 8;
-    static constexpr int CW = 8;
-    using elem = _Float16;
-    using frag = half8;
-    __device__ static __forceinline__ floatx16 mma(frag a, frag b, floatx16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ frag pack(const float *s) {
-        frag f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = (_Float16)s[i];
-        return f;
-    }
-};
-template <> struct Mma<LM_MLP_BF16> {
-    static constexpr int G = 8;
-    static constexpr int CW = 8;
-    using elem = __bf16;
-    using frag = bf16x8;
-    __device__ static __forceinline__ floatx16 mma(frag a, frag b, floatx16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-    __device__ static __forceinline__ frag pack(const float *s) {
-        frag f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = (__bf16)s[i];
-        return f;
-    }
-};
-
-// ---- layout of the packed weight buffer (all offsets in bytes, 256-byte aligned) -----------
-struct PackLayout {
-    size_t basis, w1, b1, w2, b2, w3, b3, total;
-};
-inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-inline PackLayout pack_layout(int prec, int K) {
-    const size_t E = prec == LM_MLP_F32 ? 4 : 2;
-    PackLayout L;
-    size_t o = 0;
-    L.basis = o; o = align256(o + (size_t)32 * K * E);
-    L.w1 = o; o = align256(o + (size_t)4 * kSlots1 * 64 * E);
-    L.b1 = o; o = align256(o + 4 * 2 * 16 * sizeof(float));
-    L.w2 = o; o = align256(o + (size_t)4 * 64 * 64 * E);
-    L.b2 = o; o = align256(o + 4 * 2 * 16 * sizeof(float));
-    L.w3 = o; o = align256(o + (size_t)64 * 64 * E);
-    L.b3 = o; o = align256(o + 2 * 16 * sizeof(float));
-    L.total = o;
-    return L;
-}
-
-// product channel a lane-half reads for basis slot sigma: W consecutive channels per lane,
-// the two halves interleaved so that a sample's pair of lanes reads 2W contiguous floats
-__host__ __device__ constexpr int basis_channel(int h, int sigma, int W) { return 2 * W * (sigma / W) + W * h + sigma % W; }
-
+// ---- host-side packing ----------------------------------------------------------------------
 // column of the reference's 150-wide input row that feeds slot (h, group, v); -1 = none
 inline int input_column(int h, int grp, int v) {
     const int row = row_of(v, h);
@@ -139,33 +76,38 @@ template <> inline float to_elem<float>(float x) { return x; }
 template <> inline _Float16 to_elem<_Float16>(float x) { return (_Float16)x; }
 template <> inline __bf16 to_elem<__bf16>(float x) { return (__bf16)x; }
 
-// Writes fragments [block][step][lane][G]; value(block, i, h, sigma) gives A[row i of the block][slot]
+// Writes fragments [block][step][part][lane][G]; value(block, i, h, sigma) gives
+// A[row i of the block][slot].  parts = 2 stores (hi, lo) with hi = E(x), lo = E(x - hi).
 template <typename E, typename F>
-void pack_matrix(E *dst, int n_blocks, int n_slots, int G, F value) {
+void pack_matrix(E *dst, int n_blocks, int n_slots, int G, int parts, F value) {
     const int steps = n_slots / G;
     for (int fb = 0; fb < n_blocks; ++fb)
         for (int t = 0; t < steps; ++t)
             for (int lane = 0; lane < 64; ++lane)
                 for (int e = 0; e < G; ++e) {
                     const int i = lane % 32, h = lane / 32;
-                    dst[(((size_t)fb * steps + t) * 64 + lane) * G + e] = to_elem<E>(value(fb, i, h, t * G + e));
+                    const float x = value(fb, i, h, t * G + e);
+                    const E hi = to_elem<E>(x);
+                    const size_t base = (((size_t)fb * steps + t) * parts) * 64;
+                    dst[(base + lane) * G + e] = hi;
+                    if (parts == 2) dst[(base + 64 + lane) * G + e] = to_elem<E>(x - (float)hi);
                 }
 }
 
 template <typename E>
-void pack_all(int K, int G, int CW, const PackLayout &L, const float *basis, const float *w1, const float *b1,
-              const float *w2, const float *b2, const float *w3, const float *b3, char *out) {
-    pack_matrix<E>((E *)(out + L.basis), 1, K / 2, G, [&](int, int i, int h, int s) {
+void pack_all(int K, int G, int CW, int parts, const PackLayout &L, const float *basis, const float *w1,
+              const float *b1, const float *w2, const float *b2, const float *w3, const float *b3, char *out) {
+    pack_matrix<E>((E *)(out + L.basis), 1, K / 2, G, parts, [&](int, int i, int h, int s) {
         return i < kAppDim ? basis[(size_t)i * K + basis_channel(h, s, CW)] : 0.0f;
     });
-    pack_matrix<E>((E *)(out + L.w1), 4, kSlots1, G, [&](int fb, int i, int h, int s) {
+    pack_matrix<E>((E *)(out + L.w1), 4, kSlots1, G, parts, [&](int fb, int i, int h, int s) {
         const int col = input_column(h, s / 16, s % 16);
         return col < 0 ? 0.0f : w1[(size_t)(32 * fb + i) * kInDim + col];
     });
-    pack_matrix<E>((E *)(out + L.w2), 4, 64, G, [&](int fb, int i, int h, int s) {
+    pack_matrix<E>((E *)(out + L.w2), 4, 64, G, parts, [&](int fb, int i, int h, int s) {
         return w2[(size_t)(32 * fb + i) * kHidden + 32 * (s / 16) + row_of(s % 16, h)];
     });
-    pack_matrix<E>((E *)(out + L.w3), 1, 64, G, [&](int, int i, int h, int s) {
+    pack_matrix<E>((E *)(out + L.w3), 1, 64, G, parts, [&](int, int i, int h, int s) {
         return i < 3 ? w3[(size_t)i * kHidden + 32 * (s / 16) + row_of(s % 16, h)] : 0.0f;
     });
     float *pb1 = (float *)(out + L.b1), *pb2 = (float *)(out + L.b2), *pb3 = (float *)(out + L.b3);
@@ -180,16 +122,6 @@ void pack_all(int K, int G, int CW, const PackLayout &L, const float *basis, con
 }
 
 // ---- device side ---------------------------------------------------------------------------
-// Keeps the compiler from hoisting the weight-fragment loads of later blocks above this
-// point (fully unrolled loops would otherwise keep hundreds of fragments live and spill).
-#define LM_LOAD_FENCE() asm volatile("" ::: "memory")
-// fragments loaded ahead of their MFMAs: one group between two fences
-template <int G> struct Group { static constexpr int N = G == 1 ? 16 : 10; };
-struct PackPtrs {
-    const char *basis, *w1, *w2, *w3;
-    const float *b1, *b2, *b3;
-};
-
 __device__ __forceinline__ floatx16 load_bias(const float *b, int idx) {
     floatx16 a;
     const float4 *p = reinterpret_cast<const float4 *>(b + idx * 16);
@@ -201,288 +133,384 @@ __device__ __forceinline__ floatx16 load_bias(const float *b, int idx) {
     return a;
 }
 
+// sin and cos of x to float rounding for |x| < 8192 (three-constant Cody-Waite reduction by
+// pi/2, then the minimax polynomials on [-pi/4, pi/4]); library routines beyond that.
+__device__ __forceinline__ void sincos_f32(float x, float &s, float &c) {
+    if (fabsf(x) > 8192.0f) {
+        s = sinf(x); c = cosf(x);
+        return;
+    }
+    const float k = rintf(x * 0.636619772367581f);
+    float r = fmaf(-k, 1.5703125f, x);
+    r = fmaf(-k, 4.837512969970703125e-4f, r);
+    r = fmaf(-k, 7.54978995489188216e-8f, r);
+    const float r2 = r * r;
+    float ps = fmaf(r2, -1.9515295891e-4f, 8.3321608736e-3f);
+    ps = fmaf(ps, r2, -1.6666654611e-1f);
+    ps = fmaf(ps * r2, r, r);
+    float pc = fmaf(r2, 2.443315711809948e-5f, -1.388731625493765e-3f);
+    pc = fmaf(pc, r2, 4.166664568298827e-2f);
+    pc = fmaf(pc * r2, r2, fmaf(-0.5f, r2, 1.0f));
+    const int q = (int)k & 3;
+    const float ss = (q & 1) ? pc : ps, cc = (q & 1) ? ps : pc;
+    s = (q & 2) ? -ss : ss;
+    c = ((q + 1) & 2) ? -cc : cc;
+}
+
+// One dense layer on the wave's 32 samples: acc[fb] (+)= W[32*fb .. +32, :] x B for NB row
+// blocks.  Steps run outermost so that the NB accumulator chains are independent and each
+// B fragment is used NB times; the weight fragments of step t+1 are fetched while step t
+// multiplies, and a scheduling barrier per step keeps the compiler from hoisting more.
+template <int PREC, int NB, int T>
+__device__ __forceinline__ void dense_layer(const typename Mma<PREC>::frag *W0, int fb0, unsigned lane,
+                                            const typename Mma<PREC>::frag (*b)[Mma<PREC>::NP], floatx16 *acc) {
+    const typename Mma<PREC>::frag *W = W0 + (size_t)fb0 * T * Mma<PREC>::NP * 64;
+    using M = Mma<PREC>;
+    using frag = typename M::frag;
+    constexpr int NP = M::NP;
+    constexpr bool kPrefetch = NP == 1;  // the split mode has no registers to spare for a second buffer
+    frag cur[NB][NP], nxt[NB][NP];
+#pragma unroll
+    for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+        for (int pt = 0; pt < NP; ++pt) cur[fb][pt] = W[((fb * T + 0) * NP + pt) * 64 + lane];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (kPrefetch && t + 1 < T) {
+#pragma unroll
+            for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+                for (int pt = 0; pt < NP; ++pt) nxt[fb][pt] = W[((fb * T + t + 1) * NP + pt) * 64 + lane];
+        }
+#pragma unroll
+        for (int fb = 0; fb < NB; ++fb) {
+            acc[fb] = M::mma(cur[fb][0], b[t][0], acc[fb]);
+            if constexpr (NP == 2) {
+                acc[fb] = M::mma(cur[fb][1], b[t][0], acc[fb]);
+                acc[fb] = M::mma(cur[fb][0], b[t][1], acc[fb]);
+            }
+        }
+        if (t + 1 < T) {
+#pragma unroll
+            for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+                for (int pt = 0; pt < NP; ++pt)
+                    cur[fb][pt] = kPrefetch ? nxt[fb][pt] : W[((fb * T + t + 1) * NP + pt) * 64 + lane];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// relu(acc) of NB row blocks -> B fragments of the next layer
+template <int PREC, int NB>
+__device__ __forceinline__ void relu_to_frags(const floatx16 *acc, typename Mma<PREC>::frag (*out)[Mma<PREC>::NP]) {
+    // out points at the first fragment of the first of the NB row blocks
+    using M = Mma<PREC>;
+    constexpr int G = M::G;
+#pragma unroll
+    for (int fb = 0; fb < NB; ++fb) {
+        float hv[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) hv[v] = fmaxf(acc[fb][v], 0.0f);
+#pragma unroll
+        for (int u = 0; u < 16 / G; ++u) M::pack(hv + u * G, out[fb * (16 / G) + u]);
+    }
+}
+
 // raw[16] (lane's 16 row values, view direction already inserted) -> rgb of the lane's
 // sample in out[0..2] (meaningful on lanes with h == 0)
 template <int PREC>
-__device__ __forceinline__ void colour_network(const PackPtrs &P, const float *raw, unsigned lane, float *out) {
+__device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w1, const typename Mma<PREC>::frag *w2,
+                                               const typename Mma<PREC>::frag *w3, const float *b1, const float *b2,
+                                               const float *b3, const float *raw, unsigned lane, float *out) {
     using M = Mma<PREC>;
     using frag = typename M::frag;
-    constexpr int G = M::G;
+    constexpr int G = M::G, NP = M::NP;
+    constexpr int T1 = kSlots1 / G, T2 = 64 / G;
     const unsigned h = lane >> 5;
-    float slots[kSlots1];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const float x = raw[v];
-        float s1, c1, s2, c2;
-        if (PREC == LM_MLP_F32) {
-            s1 = sinf(x); c1 = cosf(x);
-            const float x2 = x * 2.0f;
-            s2 = sinf(x2); c2 = cosf(x2);
-        } else {
-            s1 = __sinf(x); c1 = __cosf(x);
-            s2 = 2.0f * s1 * c1; c2 = 1.0f - 2.0f * s1 * s1;
-        }
-        slots[v] = x; slots[16 + v] = s1; slots[32 + v] = c1; slots[48 + v] = s2; slots[64 + v] = c2;
-    }
-    frag bfrag[kSlots1 / G];
-#pragma unroll
-    for (int t = 0; t < kSlots1 / G; ++t) bfrag[t] = M::pack(slots + t * G);
-
-    // layer 1
-    float h1[64];
+    frag b2frag[T2][NP];
     {
-        const frag *A = reinterpret_cast<const frag *>(P.w1);
-        constexpr int T = kSlots1 / G;
+        frag bfrag[T1][NP];
+        {
+            float slots[kSlots1];
 #pragma unroll
-        for (int fb = 0; fb < 4; ++fb) {
-            floatx16 acc = load_bias(P.b1, fb * 2 + h);
-#pragma unroll
-            for (int t = 0; t < T; ++t) {
-                if (t % Group<G>::N == 0) LM_LOAD_FENCE();
-                acc = M::mma(A[(fb * T + t) * 64 + lane], bfrag[t], acc);
+            for (int v = 0; v < 16; ++v) {
+                const float x = raw[v];
+                float s1, c1;
+                if (PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2) {
+                    sincos_f32(x, s1, c1);
+                } else {
+                    s1 = __sinf(x); c1 = __cosf(x);
+                }
+                const float s2 = 2.0f * s1 * c1;
+                const float c2 = fmaf(-2.0f * s1, s1, 1.0f);
+                slots[v] = x; slots[16 + v] = s1; slots[32 + v] = c1; slots[48 + v] = s2; slots[64 + v] = c2;
             }
 #pragma unroll
-            for (int v = 0; v < 16; ++v) h1[fb * 16 + v] = fmaxf(acc[v], 0.0f);
+            for (int t = 0; t < T1; ++t) M::pack(slots + t * G, bfrag[t]);
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {  // two row blocks at a time: 32 accumulator registers
+            floatx16 acc[2];
+            acc[0] = load_bias(b1, (2 * half) * 2 + h);
+            acc[1] = load_bias(b1, (2 * half + 1) * 2 + h);
+            dense_layer<PREC, 2, T1>(w1, 2 * half, lane, bfrag, acc);
+            relu_to_frags<PREC, 2>(acc, b2frag + 2 * half * (16 / G));
         }
     }
-    // layer 2
-    constexpr int T2 = 64 / G;
-    frag b2frag[T2];
-#pragma unroll
-    for (int t = 0; t < T2; ++t) b2frag[t] = M::pack(h1 + t * G);
-    float h2[64];
+    frag b3frag[T2][NP];
     {
-        const frag *A = reinterpret_cast<const frag *>(P.w2);
 #pragma unroll
-        for (int fb = 0; fb < 4; ++fb) {
-            floatx16 acc = load_bias(P.b2, fb * 2 + h);
-#pragma unroll
-            for (int t = 0; t < T2; ++t) {
-                if (t % Group<G>::N == 0) LM_LOAD_FENCE();
-                acc = M::mma(A[(fb * T2 + t) * 64 + lane], b2frag[t], acc);
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) h2[fb * 16 + v] = fmaxf(acc[v], 0.0f);
+        for (int half = 0; half < 2; ++half) {
+            floatx16 acc[2];
+            acc[0] = load_bias(b2, (2 * half) * 2 + h);
+            acc[1] = load_bias(b2, (2 * half + 1) * 2 + h);
+            dense_layer<PREC, 2, T2>(w2, 2 * half, lane, b2frag, acc);
+            relu_to_frags<PREC, 2>(acc, b3frag + 2 * half * (16 / G));
         }
     }
-    // layer 3 (rows 0..2 real)
-    {
-        const frag *A = reinterpret_cast<const frag *>(P.w3);
-        floatx16 acc = load_bias(P.b3, h);
+    floatx16 acc3[1];
+    acc3[0] = load_bias(b3, h);
+    dense_layer<PREC, 1, T2>(w3, 0, lane, b3frag, acc3);
 #pragma unroll
-        for (int t = 0; t < T2; ++t) {
-            if (t % Group<G>::N == 0) LM_LOAD_FENCE();
-            acc = M::mma(A[t * 64 + lane], M::pack(h2 + t * G), acc);
-        }
-#pragma unroll
-        for (int k = 0; k < 3; ++k) out[k] = 1.0f / (1.0f + expf(-acc[k]));
-    }
+    for (int k = 0; k < 3; ++k) out[k] = 1.0f / (1.0f + expf(-acc3[0][k]));
 }
 
-// basis_mat on 32 samples: products row of the lane's sample -> 16 row values per lane
-template <int PREC>
-__device__ __forceinline__ floatx16 basis_project(const PackPtrs &P, int K, const float *__restrict__ row, unsigned lane) {
+template <int PREC> struct LdsPlan {
     using M = Mma<PREC>;
-    using frag = typename M::frag;
-    constexpr int G = M::G, CW = M::CW;
-    const unsigned h = lane >> 5;
-    const frag *A = reinterpret_cast<const frag *>(P.basis);
-    floatx16 acc;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-    // per iteration a lane consumes CW consecutive channels = CW/G MFMA steps
-    const int iters = (K / 2) / CW;
-    for (int it = 0; it < iters; ++it) {
-        float c[CW];
-        const float4 *src = reinterpret_cast<const float4 *>(row + 2 * CW * it + CW * h);
-#pragma unroll
-        for (int i = 0; i < CW / 4; ++i) {
-            float4 t = src[i];
-            c[4 * i] = t.x; c[4 * i + 1] = t.y; c[4 * i + 2] = t.z; c[4 * i + 3] = t.w;
-        }
-#pragma unroll
-        for (int u = 0; u < CW / G; ++u) acc = M::mma(A[(it * (CW / G) + u) * 64 + lane], M::pack(c + u * G), acc);
-    }
-    return acc;
-}
+    static constexpr size_t kW1 = (size_t)4 * kSlots1 * 64 * sizeof(typename M::elem) * M::NP;
+    static constexpr size_t kW2 = (size_t)4 * 64 * 64 * sizeof(typename M::elem) * M::NP;
+    static constexpr size_t kW3 = (size_t)64 * 64 * sizeof(typename M::elem) * M::NP;
+    static constexpr bool kW3InLds = (kW1 + kW2 + kW3) <= 96 * 1024;
+    static constexpr size_t kBytes = kW1 + kW2 + (kW3InLds ? kW3 : 0);
+};
 
-__device__ __forceinline__ PackPtrs make_ptrs(const char *packed, PackLayout L) {
-    PackPtrs P;
-    P.basis = packed + L.basis; P.w1 = packed + L.w1; P.w2 = packed + L.w2; P.w3 = packed + L.w3;
-    P.b1 = (const float *)(packed + L.b1); P.b2 = (const float *)(packed + L.b2); P.b3 = (const float *)(packed + L.b3);
-    return P;
-}
-
-// feat [M,27], view [M,3] -> rgb [M,3]
 template <int PREC>
-__global__ __launch_bounds__(kBlock) void k_mlp_feat(const char *__restrict__ packed, PackLayout L,
-                                                     const float *__restrict__ feat, const float *__restrict__ view,
-                                                     uint64_t M, float *__restrict__ rgb) {
-    const PackPtrs P = make_ptrs(packed, L);
+__device__ __forceinline__ void stage_weights(char *lds, const char *packed, const PackLayout &L) {
+    using P = LdsPlan<PREC>;
+    const uint4 *s1 = reinterpret_cast<const uint4 *>(packed + L.w1);
+    const uint4 *s2 = reinterpret_cast<const uint4 *>(packed + L.w2);
+    const uint4 *s3 = reinterpret_cast<const uint4 *>(packed + L.w3);
+    uint4 *d = reinterpret_cast<uint4 *>(lds);
+    for (size_t i = threadIdx.x; i < P::kW1 / 16; i += blockDim.x) d[i] = s1[i];
+    d += P::kW1 / 16;
+    for (size_t i = threadIdx.x; i < P::kW2 / 16; i += blockDim.x) d[i] = s2[i];
+    d += P::kW2 / 16;
+    if (P::kW3InLds)
+        for (size_t i = threadIdx.x; i < P::kW3 / 16; i += blockDim.x) d[i] = s3[i];
+    __syncthreads();
+}
+
+// Colour network over a list of rows.
+//   MODE 0: feat [M,27] and view [M,3] given per row (isolated network)
+//   MODE 1: feat [n,27] per appearance slot, view direction = direction of the slot's ray
+template <int PREC, int MODE>
+__global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restrict__ packed, PackLayout L,
+                                                   const float *__restrict__ feat, const float *__restrict__ view,
+                                                   uint64_t M_host, const uint32_t *__restrict__ count, int S,
+                                                   const uint32_t *__restrict__ app_idx, float *__restrict__ rgb) {
+    extern __shared__ __align__(16) char lds[];
+    using Mm = Mma<PREC>;
+    using frag = typename Mm::frag;
+    using P = LdsPlan<PREC>;
+    stage_weights<PREC>(lds, packed, L);
+    const frag *w1 = reinterpret_cast<const frag *>(lds);
+    const frag *w2 = reinterpret_cast<const frag *>(lds + P::kW1);
+    const frag *w3 = P::kW3InLds ? reinterpret_cast<const frag *>(lds + P::kW1 + P::kW2)
+                                 : reinterpret_cast<const frag *>(packed + L.w3);
+    const float *b1 = (const float *)(packed + L.b1), *b2 = (const float *)(packed + L.b2),
+                *b3 = (const float *)(packed + L.b3);
     const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
+    const uint64_t M = MODE == 0 ? M_host : (uint64_t)*count;
     const uint64_t n_tiles = (M + 31) / 32;
-    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * (kBlock / LM_WAVE) + threadIdx.x / LM_WAVE;
-    const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / LM_WAVE);
+    const unsigned wpb = MlpBlock<PREC>::N / LM_WAVE;
+    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * wpb + threadIdx.x / LM_WAVE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * wpb;
     for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
         const uint64_t p = tile * 32 + j;
         const bool live = p < M;
         const uint64_t pc = live ? p : M - 1;
+        const float *vsrc = MODE == 0 ? view + pc * 3 : view + 6 * (size_t)(app_idx[pc] / (uint32_t)S) + 3;
         float raw[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int row = row_of(v, (int)h);
             float x = 0.0f;
             if (row < kAppDim) x = feat[pc * kAppDim + row];
-            else if (row >= 28 && row <= 30) x = view[pc * 3 + (row - 28)];
+            else if (row >= 28 && row <= 30) x = vsrc[row - 28];
             raw[v] = x;
         }
         float out[3];
-        colour_network<PREC>(P, raw, lane, out);
+        colour_network<PREC>(w1, w2, w3, b1, b2, b3, raw, lane, out);
         if (live && h == 0) {
             rgb[p * 3 + 0] = out[0]; rgb[p * 3 + 1] = out[1]; rgb[p * 3 + 2] = out[2];
         }
     }
 }
 
-// products [M,K] -> feat [M,27]
+// products [M,K] -> feat [M,27] (stand-alone basis_mat; fragments straight from global memory)
 template <int PREC>
-__global__ __launch_bounds__(kBlock) void k_basis(const char *__restrict__ packed, PackLayout L, int K,
-                                                  const float *__restrict__ products, uint64_t M,
-                                                  float *__restrict__ feat) {
-    const PackPtrs P = make_ptrs(packed, L);
+__global__ __launch_bounds__(256) void k_basis(const char *__restrict__ packed, PackLayout L, int K,
+                                               const float *__restrict__ products, uint64_t M_host,
+                                               const uint32_t *__restrict__ count, float *__restrict__ feat) {
+    const uint64_t M = count ? (uint64_t)*count : M_host;
+    using Mm = Mma<PREC>;
+    using frag = typename Mm::frag;
+    constexpr int G = Mm::G, CW = Mm::CW, NP = Mm::NP;
     const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
     const uint64_t n_tiles = (M + 31) / 32;
-    const uint64_t wave_id = (uint64_t)blockIdx.x * (kBlock / LM_WAVE) + threadIdx.x / LM_WAVE;
-    const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / LM_WAVE);
+    const uint64_t wave_id = (uint64_t)blockIdx.x * 4 + threadIdx.x / LM_WAVE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * 4;
+    const frag *A = reinterpret_cast<const frag *>(packed + L.basis);
     for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
         const uint64_t p = tile * 32 + j;
         const bool live = p < M;
-        const uint64_t pc = live ? p : M - 1;
-        const floatx16 acc = basis_project<PREC>(P, K, products + pc * (uint64_t)K, lane);
+        const float *row = products + (live ? p : M - 1) * (uint64_t)K;
+        floatx16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+        const int iters = (K / 2) / CW;
+        for (int it = 0; it < iters; ++it) {
+            float c[CW];
+            const float4 *src = reinterpret_cast<const float4 *>(row + 2 * CW * it + CW * h);
+#pragma unroll
+            for (int i = 0; i < CW / 4; ++i) {
+                float4 t = src[i];
+                c[4 * i] = t.x; c[4 * i + 1] = t.y; c[4 * i + 2] = t.z; c[4 * i + 3] = t.w;
+            }
+#pragma unroll
+            for (int u = 0; u < CW / G; ++u) {
+                frag b[NP];
+                Mm::pack(c + u * G, b);
+                const int t = it * (CW / G) + u;
+                const frag a0 = A[(t * NP) * 64 + lane];
+                acc = Mm::mma(a0, b[0], acc);
+                if constexpr (NP == 2) {
+                    const frag a1 = A[(t * NP + 1) * 64 + lane];
+                    acc = Mm::mma(a1, b[0], acc);
+                    acc = Mm::mma(a0, b[1], acc);
+                }
+            }
+        }
         if (live) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const int row = row_of(v, (int)h);
-                if (row < kAppDim) feat[p * kAppDim + row] = acc[v];
+                const int r = row_of(v, (int)h);
+                if (r < kAppDim) feat[p * kAppDim + r] = acc[v];
             }
         }
     }
 }
 
-// inside the render: products [n_app,K] + ray directions -> rgb [n_app,3]
-template <int PREC>
-__global__ __launch_bounds__(kBlock) void k_app_colour(const char *__restrict__ packed, PackLayout L, int K, int S,
-                                                       const float *__restrict__ products,
-                                                       const float *__restrict__ rays,
-                                                       const uint32_t *__restrict__ app_idx,
-                                                       const uint32_t *__restrict__ count, float *__restrict__ rgb) {
-    const PackPtrs P = make_ptrs(packed, L);
-    const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
-    const uint64_t M = *count;
-    const uint64_t n_tiles = (M + 31) / 32;
-    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * (kBlock / LM_WAVE) + threadIdx.x / LM_WAVE;
-    const uint64_t n_waves = (uint64_t)gridDim.x * (kBlock / LM_WAVE);
-    for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
-        const uint64_t p = tile * 32 + j;
-        const bool live = p < M;
-        const uint64_t pc = live ? p : M - 1;
-        const floatx16 acc = basis_project<PREC>(P, K, products + pc * (uint64_t)K, lane);
-        float raw[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) raw[v] = acc[v];
-        if (h == 1) {
-            const uint32_t r = app_idx[pc] / (uint32_t)S;
-            raw[12] = rays[6 * (size_t)r + 3]; raw[13] = rays[6 * (size_t)r + 4]; raw[14] = rays[6 * (size_t)r + 5];
-        }
-        raw[15] = 0.0f;
-        float out[3];
-        colour_network<PREC>(P, raw, lane, out);
-        if (live && h == 0) {
-            rgb[p * 3 + 0] = out[0]; rgb[p * 3 + 1] = out[1]; rgb[p * 3 + 2] = out[2];
-        }
+template <int PREC, int MODE>
+int launch_mlp(const void *packed, int K, const float *feat, const float *view, uint64_t M, const uint32_t *count,
+               int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t stream) {
+    const PackLayout L = pack_layout(PREC, K);
+    const size_t lds = LdsPlan<PREC>::kBytes;
+    static thread_local bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mlp<PREC, MODE>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) LM_FAIL(LM_ERR_LAUNCH, "k_mlp: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        configured = true;
+    }
+    hipLaunchKernelGGL((k_mlp<PREC, MODE>), dim3(grid), dim3(MlpBlock<PREC>::N), lds, stream, (const char *)packed, L, feat, view,
+                       M, count, S, app_idx, rgb);
+    LM_CHECK_LAUNCH("k_mlp");
+    return LM_OK;
+}
+
+template <int MODE>
+int dispatch_mlp(int prec, const void *packed, int K, const float *feat, const float *view, uint64_t M,
+                 const uint32_t *count, int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t st) {
+    switch (prec) {
+        case LM_MLP_F32: return launch_mlp<LM_MLP_F32, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
+        case LM_MLP_F16: return launch_mlp<LM_MLP_F16, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
+        case LM_MLP_BF16: return launch_mlp<LM_MLP_BF16, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
+        default: return launch_mlp<LM_MLP_F16X2, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
     }
 }
 
 }  // namespace
 
-static int check_prec(int prec) {
-    LM_REQUIRE(prec == LM_MLP_F32 || prec == LM_MLP_F16 || prec == LM_MLP_BF16, "unknown colour-network precision %d", prec);
+int lm_check_prec(int prec) {
+    LM_REQUIRE(prec == LM_MLP_F32 || prec == LM_MLP_F16 || prec == LM_MLP_BF16 || prec == LM_MLP_F16X2,
+               "unknown colour-network precision %d", prec);
     return LM_OK;
 }
-static int check_K(int K) {
+int lm_check_K(int K) {
     LM_REQUIRE(K >= 16 && K % 16 == 0 && K <= 4096, "basis_mat input width %d must be a multiple of 16 in 16..4096", K);
     return LM_OK;
 }
 
 extern "C" size_t lm_mlp_packed_bytes(int32_t prec, int32_t K_basis) {
-    if (check_prec(prec) || check_K(K_basis)) return 0;
+    if (lm_check_prec(prec) || lm_check_K(K_basis)) return 0;
     return pack_layout(prec, K_basis).total;
 }
 
 extern "C" int lm_mlp_pack(int32_t prec, int32_t K, const float *basis, const float *w1, const float *b1,
                            const float *w2, const float *b2, const float *w3, const float *b3, void *packed_out) {
-    if (int rc = check_prec(prec)) return rc;
-    if (int rc = check_K(K)) return rc;
+    if (int rc = lm_check_prec(prec)) return rc;
+    if (int rc = lm_check_K(K)) return rc;
     LM_REQUIRE(basis && w1 && w2 && w3 && packed_out, "null weight pointer");
     const PackLayout L = pack_layout(prec, K);
     memset(packed_out, 0, L.total);
     char *out = (char *)packed_out;
-    if (prec == LM_MLP_F32) pack_all<float>(K, 1, 4, L, basis, w1, b1, w2, b2, w3, b3, out);
-    else if (prec == LM_MLP_F16) pack_all<_Float16>(K, 8, 8, L, basis, w1, b1, w2, b2, w3, b3, out);
-    else pack_all<__bf16>(K, 8, 8, L, basis, w1, b1, w2, b2, w3, b3, out);
+    if (prec == LM_MLP_F32) pack_all<float>(K, 1, 4, 1, L, basis, w1, b1, w2, b2, w3, b3, out);
+    else if (prec == LM_MLP_F16) pack_all<_Float16>(K, 8, 8, 1, L, basis, w1, b1, w2, b2, w3, b3, out);
+    else if (prec == LM_MLP_BF16) pack_all<__bf16>(K, 8, 8, 1, L, basis, w1, b1, w2, b2, w3, b3, out);
+    else pack_all<_Float16>(K, 8, 8, 2, L, basis, w1, b1, w2, b2, w3, b3, out);
     return LM_OK;
 }
 
-#define LM_DISPATCH_PREC(prec, KERNEL, grid, stream, ...)                                                         \
-    do {                                                                                                          \
-        if ((prec) == LM_MLP_F32)                                                                                 \
-            hipLaunchKernelGGL(KERNEL<LM_MLP_F32>, dim3(grid), dim3(kBlock), 0, (hipStream_t)(stream), __VA_ARGS__); \
-        else if ((prec) == LM_MLP_F16)                                                                            \
-            hipLaunchKernelGGL(KERNEL<LM_MLP_F16>, dim3(grid), dim3(kBlock), 0, (hipStream_t)(stream), __VA_ARGS__); \
-        else                                                                                                      \
-            hipLaunchKernelGGL(KERNEL<LM_MLP_BF16>, dim3(grid), dim3(kBlock), 0, (hipStream_t)(stream), __VA_ARGS__); \
-    } while (0)
-
-static unsigned wave_tile_grid(uint64_t M) {
-    const uint64_t tiles = (M + 31) / 32, blocks = (tiles + 3) / 4;
-    return (unsigned)std::min<uint64_t>(std::max<uint64_t>(blocks, 1), (uint64_t)lm_persistent_blocks(2));
+static unsigned mlp_grid(uint64_t M) {
+    const uint64_t tiles = (M + 31) / 32, wpb = 4, blocks = (tiles + wpb - 1) / wpb;
+    return (unsigned)std::min<uint64_t>(std::max<uint64_t>(blocks, 1), (uint64_t)lm_persistent_blocks(1));
 }
 
 extern "C" int lm_mlp(int32_t prec, const void *packed, int32_t K, const float *feat, const float *view, int64_t M,
                       float *rgb, void *stream) {
-    if (int rc = check_prec(prec)) return rc;
-    if (int rc = check_K(K)) return rc;
+    if (int rc = lm_check_prec(prec)) return rc;
+    if (int rc = lm_check_K(K)) return rc;
     LM_REQUIRE(M >= 0, "negative count");
     if (M == 0) return LM_OK;
     LM_REQUIRE(packed && feat && view && rgb && lm_aligned16(packed), "null or misaligned buffer");
+    return dispatch_mlp<0>(prec, packed, K, feat, view, (uint64_t)M, nullptr, 1, nullptr, rgb, mlp_grid((uint64_t)M),
+                           (hipStream_t)stream);
+}
+
+// products [M,K] -> feat [M,27]; M from the host, or from *count when count != NULL
+int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
+                    float *feat, hipStream_t st) {
+    if (int rc = lm_check_prec(prec)) return rc;
+    if (int rc = lm_check_K(K)) return rc;
+    LM_REQUIRE(packed && products && feat && lm_aligned16(packed) && lm_aligned16(products), "null or misaligned buffer");
     const PackLayout L = pack_layout(prec, K);
-    LM_DISPATCH_PREC(prec, k_mlp_feat, wave_tile_grid((uint64_t)M), stream, (const char *)packed, L, feat, view, (uint64_t)M, rgb);
-    LM_CHECK_LAUNCH("k_mlp_feat");
+    const uint64_t tiles = (M + 31) / 32;
+    const unsigned grid = count ? (unsigned)lm_persistent_blocks(4)
+                                : (unsigned)std::min<uint64_t>(std::max<uint64_t>((tiles + 3) / 4, 1), (uint64_t)lm_persistent_blocks(4));
+    switch (prec) {
+        case LM_MLP_F32: hipLaunchKernelGGL(k_basis<LM_MLP_F32>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
+        case LM_MLP_F16: hipLaunchKernelGGL(k_basis<LM_MLP_F16>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
+        case LM_MLP_BF16: hipLaunchKernelGGL(k_basis<LM_MLP_BF16>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
+        default: hipLaunchKernelGGL(k_basis<LM_MLP_F16X2>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
+    }
+    LM_CHECK_LAUNCH("k_basis");
     return LM_OK;
 }
 
 extern "C" int lm_basis(int32_t prec, const void *packed, int32_t K, const float *products, int64_t M, float *feat,
                         void *stream) {
-    if (int rc = check_prec(prec)) return rc;
-    if (int rc = check_K(K)) return rc;
     LM_REQUIRE(M >= 0, "negative count");
     if (M == 0) return LM_OK;
-    LM_REQUIRE(packed && products && feat && lm_aligned16(packed) && lm_aligned16(products), "null or misaligned buffer");
-    const PackLayout L = pack_layout(prec, K);
-    LM_DISPATCH_PREC(prec, k_basis, wave_tile_grid((uint64_t)M), stream, (const char *)packed, L, (int)K, products, (uint64_t)M, feat);
-    LM_CHECK_LAUNCH("k_basis");
-    return LM_OK;
+    return lm_launch_basis(prec, packed, K, products, (uint64_t)M, nullptr, feat, (hipStream_t)stream);
 }
 
-// used by lm_render
-int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *products, const float *rays,
+// used by lm_render: feat [n_app,27] + ray directions -> rgb [n_app,3]
+int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *feat, const float *rays,
                          const uint32_t *app_idx, const uint32_t *count, float *rgb, hipStream_t stream) {
-    if (int rc = check_prec(prec)) return rc;
-    if (int rc = check_K(K)) return rc;
+    if (int rc = lm_check_prec(prec)) return rc;
+    if (int rc = lm_check_K(K)) return rc;
     LM_REQUIRE(packed && lm_aligned16(packed), "packed colour-network weights are null or misaligned");
-    const PackLayout L = pack_layout(prec, K);
-    const unsigned grid = (unsigned)lm_persistent_blocks(2);
-    LM_DISPATCH_PREC(prec, k_app_colour, grid, stream, (const char *)packed, L, K, S, products, rays, app_idx, count, rgb);
-    LM_CHECK_LAUNCH("k_app_colour");
-    return LM_OK;
+    return dispatch_mlp<1>(prec, packed, K, feat, rays, 0, count, S, app_idx, rgb, (unsigned)lm_persistent_blocks(1), stream);
 }

@@ -201,7 +201,10 @@ class GridNeRFHIP:
     def workspace(self, n_rays: int, S: int) -> torch.Tensor:
         """Device workspace for chunks of up to n_rays rays; grown on demand and reused
         (the role of allocate_tensors, dist_render/kernel/cuda_render_extend.py:35-159)."""
-        need = self.lib.lm_render_workspace_bytes(n_rays, S, self.K_app)
+        m = self._model_struct(S, True)
+        need = self.lib.lm_render_workspace_bytes(C.byref(m), n_rays)
+        if need == 0:
+            raise L.LandmarkError(self.lib.lm_last_error().decode())
         if self._ws is None or self._ws.numel() < need:
             self._ws = None
             self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
@@ -225,22 +228,34 @@ class GridNeRFHIP:
         if rays.dim() != 2 or rays.shape[1] != 6:
             raise ValueError(f"rays_chunk must be [N,6], got {tuple(rays.shape)}")
         N = rays.shape[0]
-        S = self._samples_for(N_samples)
         rgb = torch.empty((N, 3), dtype=torch.float32, device=self.device)
         depth = torch.empty((N,), dtype=torch.float32, device=self.device)
-        if N:
-            ws = self.workspace(N, S)
-            m = self._model_struct(S, white_bg)
-            L.check(
-                self.lib.lm_render(
-                    C.byref(m), rays.data_ptr(), N, ws.data_ptr(), ws.numel(), rgb.data_ptr(), depth.data_ptr(),
-                    self.counters.data_ptr(), L.current_stream(),
-                ),
-                "lm_render",
-            )
+        self.render_into(rays, rgb, depth, white_bg=white_bg, N_samples=N_samples)
         return {"rgb_map": rgb, "depth_map": depth}, {}
 
     __call__ = forward
+
+    def render_into(self, rays, rgb, depth, white_bg=True, N_samples=-1, counters=None, events=None):
+        """lm_render on device tensors the caller owns.  `counters`: int32[8] device tensor
+        receiving the chunk's sample counts; `events`: 7 recorded torch.cuda.Event objects
+        (enable_timing=True) re-recorded around the stages on the current stream."""
+        N = rays.shape[0]
+        if N == 0:
+            return
+        S = self._samples_for(N_samples)
+        ws = self.workspace(N, S)
+        m = self._model_struct(S, white_bg)
+        if events is not None:
+            for i, e in enumerate(events):
+                m.events[i] = e.cuda_event
+        cnt = self.counters if counters is None else counters
+        L.check(
+            self.lib.lm_render(
+                C.byref(m), rays.data_ptr(), N, ws.data_ptr(), ws.numel(), rgb.data_ptr(), depth.data_ptr(),
+                cnt.data_ptr(), L.current_stream(),
+            ),
+            "lm_render",
+        )
 
     def last_counts(self) -> Dict[str, int]:
         """Valid / appearance sample counts of the last chunk (synchronises)."""
@@ -343,14 +358,14 @@ class GridNeRFHIP:
 
     @torch.no_grad()
     def weights(self, cull, sigma, term_eps=None):
-        """Part 4 on a `sample_cull` result: dense weights, appearance mask, acc, depth."""
+        """Part 4 on a `sample_cull` result: dense weights, appearance list and mask, acc, depth."""
         rays, S = cull["rays"], cull["S"]
         N = rays.shape[0]
-        steps = (S + 63) // 64
         dev = self.device
         weight = torch.zeros((N, S), dtype=torch.float32, device=dev)
-        app_bits = torch.zeros((N, steps), dtype=torch.int64, device=dev)
-        app_base = torch.zeros((N, steps), dtype=torch.int32, device=dev)
+        w_valid = torch.zeros(max(cull["n_valid"], 1), dtype=torch.float32, device=dev)
+        app_first = torch.zeros(N, dtype=torch.int32, device=dev)
+        app_cnt = torch.zeros(N, dtype=torch.int32, device=dev)
         app_idx = torch.zeros(max(N * S, 1), dtype=torch.int32, device=dev)
         app_w = torch.zeros(max(N * S, 1), dtype=torch.float32, device=dev)
         acc = torch.zeros(N, dtype=torch.float32, device=dev)
@@ -363,18 +378,37 @@ class GridNeRFHIP:
             self.lib.lm_weights(
                 C.byref(g), rays.data_ptr(), N, cull["bitmap"].data_ptr(), cull["word_prefix"].data_ptr(), sig.data_ptr(),
                 self.p.distance_scale, self.p.rayMarch_weight_thres, self.term_eps if term_eps is None else term_eps,
-                weight.data_ptr(), app_bits.data_ptr(), app_base.data_ptr(), app_idx.data_ptr(), app_w.data_ptr(),
-                acc.data_ptr(), depth.data_ptr(), cnt.data_ptr(), L.current_stream(),
+                w_valid.data_ptr(), weight.data_ptr(), app_first.data_ptr(), app_cnt.data_ptr(), app_idx.data_ptr(),
+                app_w.data_ptr(), acc.data_ptr(), depth.data_ptr(), cnt.data_ptr(), L.current_stream(),
             ),
             "lm_weights",
         )
         n_app = int(cnt[L.LM_STAT_N_APP].item()) & 0xFFFFFFFF
-        bits = (app_bits[:, :, None] >> torch.arange(64, device=dev)) & 1
-        app_mask = bits.reshape(N, steps * 64)[:, :S].bool()
+        idx = app_idx[:n_app].long() & 0xFFFFFFFF
+        app_mask = torch.zeros(N * S, dtype=torch.bool, device=dev)
+        app_mask[idx] = True
         return {
-            "weight": weight, "app_mask": app_mask, "acc_map": acc, "depth_map": depth, "n_app": n_app,
-            "app_idx": app_idx[:n_app].long() & 0xFFFFFFFF, "app_w": app_w[:n_app],
+            "weight": weight, "app_mask": app_mask.view(N, S), "acc_map": acc, "depth_map": depth, "n_app": n_app,
+            "app_idx": idx, "app_w": app_w[:n_app], "app_first": app_first.long(), "app_cnt": app_cnt.long(),
+            "w_valid": w_valid[: cull["n_valid"]], "counters": cnt, "app_idx_raw": app_idx,
         }
+
+    @torch.no_grad()
+    def app_features_list(self, cull, wres, precision=None):
+        """Fused gather + basis_mat over the appearance list of a `weights` result -> [n_app,27]."""
+        old = self.mlp_precision
+        self.mlp_precision = precision or old
+        try:
+            m = self._model_struct(cull["S"], True)
+            feat = torch.zeros((max(wres["n_app"], 1), 27), dtype=torch.float32, device=self.device)
+            L.check(
+                self.lib.lm_app_features(C.byref(m), cull["rays"].data_ptr(), wres["app_idx_raw"].data_ptr(),
+                                         wres["counters"].data_ptr(), feat.data_ptr(), L.current_stream()),
+                "lm_app_features",
+            )
+        finally:
+            self.mlp_precision = old
+        return feat[: wres["n_app"]]
 
 
 def from_reference_model(model, **kw) -> GridNeRFHIP:

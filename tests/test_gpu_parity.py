@@ -130,7 +130,7 @@ def test_gather_closed_forms(gpu_lib):
 
 
 # ------------------------------------------------------------------------------------ part 3
-@pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16", 4e-3), ("bf16", 3e-2)])
+@pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16x2", 3e-6), ("f16", 4e-3), ("bf16", 3e-2)])
 def test_colour_network(gpu_lib, prec, tol):
     p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48)
     g = torch.Generator().manual_seed(6)
@@ -141,7 +141,7 @@ def test_colour_network(gpu_lib, prec, tol):
         assert (got - ref).abs().max().item() < tol, (M, prec)
 
 
-@pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16", 2e-3)])
+@pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16x2", 3e-6), ("f16", 2e-3)])
 def test_basis_projection(gpu_lib, prec, tol):
     p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48, ndims=3, resMode=(1, 2))
     g = torch.Generator().manual_seed(6)
@@ -169,12 +169,35 @@ def test_weights_against_raw2alpha(gpu_lib):
     assert torch.allclose(w["depth_map"].cpu(), ref["depth_map"], atol=2e-5)
     band = (ref["weight"] - p.rayMarch_weight_thres).abs() < 1e-6
     assert torch.equal(w["app_mask"].cpu() | band, ref["app_mask"] | band)
-    assert w["n_app"] == int(w["app_mask"].sum())
-    # the appearance list holds exactly the masked samples, each with its weight
+    assert w["n_app"] == int(w["app_mask"].sum()) == int(w["app_cnt"].sum())
+    # the compact weights are the dense ones at the valid samples
+    assert torch.equal(w["w_valid"], w["weight"].reshape(-1)[cull["valid_idx"]])
+    # a ray's slots are contiguous, in sample order, and hold exactly its masked samples with their weights
     flat = w["app_mask"].reshape(-1).nonzero()[:, 0]
     order = torch.argsort(w["app_idx"])
     assert torch.equal(w["app_idx"][order], flat)
     assert torch.equal(w["app_w"][order], w["weight"].reshape(-1)[flat])
+    S = cull["S"]
+    for r in w["app_cnt"].nonzero()[:50, 0].tolist():
+        first, n = int(w["app_first"][r]), int(w["app_cnt"][r])
+        seg = w["app_idx"][first : first + n]
+        assert torch.equal(seg, w["app_mask"][r].nonzero()[:, 0] + r * S)
+
+
+@pytest.mark.parametrize("prec,tol", [("f16x2", 5e-6), ("f16", 5e-3), ("bf16", 4e-2)])
+def test_fused_appearance_features(gpu_lib, prec, tol):
+    """gather + basis_mat over the appearance list against the oracle's compute_appfeature"""
+    p = _scene(S=64, resMode=(1, 2), thre=0.0)
+    rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    m = _model(p, mlp_precision=prec)
+    cull = m.sample_cull(rays)
+    w = m.weights(cull, m.density_valid(cull))
+    assert w["n_app"] > 100
+    feat = m.app_features_list(cull, w).cpu()
+    pts, _, _ = O.sample_ray_within_hull(p, rays[:, :3], rays[:, 3:6], 64)
+    xyz = O.normalize_coord(p, pts).reshape(-1, 3)[w["app_idx"].cpu()]
+    ref = O.app_feature(p, xyz)
+    assert (feat - ref).abs().max().item() < tol
 
 
 # ------------------------------------------------------------------------------------ whole path
@@ -226,6 +249,7 @@ def test_render_c1_tiny_config(gpu_lib):
 def test_render_16bit_network_and_fp16_tables(gpu_lib):
     p = _scene(S=64)
     rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    _check_render(p, rays, RGB_TOL_F32, mlp_precision="f16x2")
     _check_render(p, rays, RGB_TOL_16, mlp_precision="f16")
     _check_render(p, rays, 3e-2, mlp_precision="bf16")
     _check_render(O.to_fp16_features(p), rays, RGB_TOL_16)

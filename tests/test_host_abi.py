@@ -50,7 +50,6 @@ def test_argument_validation_returns_status_not_abort(lib):
     assert rc == -1 and b"S must be positive" in lib.lm_last_error()
     assert lib.lm_mlp_packed_bytes(7, 144) == 0
     assert lib.lm_mlp_packed_bytes(L.LM_MLP_F32, 100) == 0  # K not a multiple of 16
-    assert lib.lm_render_workspace_bytes(0, 128, 144) == 0
     pl = (L.LmPlane * 1)()
     rc = lib.lm_gather_density_xyz(pl, 1, None, 10, None, None)
     assert rc == -1 and b"null table" in lib.lm_last_error()
@@ -58,11 +57,30 @@ def test_argument_validation_returns_status_not_abort(lib):
     assert lib.lm_relayout_nchw_to_hwc(None, None, 4, 4, 4, 0, None) == -1
 
 
+def _host_model(S=128, C=48, n=3):
+    """An lm_model good enough for size queries (pointers are never dereferenced on the host)."""
+    m = L.LmModel()
+    m.geom.S, m.geom.sampler = S, L.LM_SAMPLER_HULL
+    m.geom.tab_a = m.geom.tab_t = 16
+    m.n_planes = n
+    for k in range(n):
+        for arr, c in ((m.density, 16), (m.app, C)):
+            arr[k].plane = arr[k].line = 16
+            arr[k].H = arr[k].W = arr[k].Len = 8
+            arr[k].C = c
+    m.mlp_prec = L.LM_MLP_F16X2
+    return m
+
+
 def test_workspace_size_grows_with_chunk(lib):
-    a = lib.lm_render_workspace_bytes(1024, 128, 144)
-    b = lib.lm_render_workspace_bytes(2048, 128, 144)
-    c = lib.lm_render_workspace_bytes(2048, 128, 432)
-    assert 0 < a < b < c
+    m = _host_model()
+    a = lib.lm_render_workspace_bytes(C.byref(m), 1024)
+    b = lib.lm_render_workspace_bytes(C.byref(m), 2048)
+    assert 0 < a < b
+    assert lib.lm_render_workspace_bytes(C.byref(m), 0) == 0
+    # channel counts the fused appearance kernel does not cover need the product matrix as well
+    c = lib.lm_render_workspace_bytes(C.byref(_host_model(C=12, n=4)), 2048)
+    assert c > b
 
 
 # ---------------------------------------------------------------- packing replay
@@ -71,7 +89,7 @@ def row_of(v, h):
 
 
 def _layout(prec, K):
-    E = 4 if prec == L.LM_MLP_F32 else 2
+    E = (4 if prec == L.LM_MLP_F32 else 2) * (2 if prec == L.LM_MLP_F16X2 else 1)
     al = lambda x: (x + 255) & ~255
     o = 0
     out = {}
@@ -82,11 +100,11 @@ def _layout(prec, K):
     return out
 
 
-def _frags(buf, off, n_blocks, n_slots, G, dt):
+def _frags(buf, off, n_blocks, n_slots, G, dt, parts=1):
     steps = n_slots // G
-    n = n_blocks * steps * 64 * G
-    a = np.frombuffer(buf, dtype=dt, count=n, offset=off).astype(np.float32)
-    return a.reshape(n_blocks, steps, 64, G)
+    n = n_blocks * steps * parts * 64 * G
+    a = np.frombuffer(buf, dtype=dt, count=n, offset=off).astype(np.float64)
+    return a.reshape(n_blocks, steps, parts, 64, G).sum(axis=2)  # hi + lo
 
 
 def _mma_layer(A, slots):
@@ -107,7 +125,7 @@ def _regs(D):
     return out.reshape(n, 2, nb * 16)
 
 
-@pytest.mark.parametrize("prec,dt,tol", [(L.LM_MLP_F32, np.float32, 2e-6), (L.LM_MLP_F16, np.float16, 3e-3)])
+@pytest.mark.parametrize("prec,dt,tol", [(L.LM_MLP_F32, np.float32, 2e-6), (L.LM_MLP_F16, np.float16, 3e-3), (L.LM_MLP_F16X2, np.float16, 2e-6)])
 def test_packed_weights_replay_matches_oracle(lib, prec, dt, tol):
     p = scenes.make_params(seed=11, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=16, ndims=3, resMode=(1,))
     K = 48
@@ -121,6 +139,9 @@ def test_packed_weights_replay_matches_oracle(lib, prec, dt, tol):
     buf = host.tobytes()
     G = 1 if prec == L.LM_MLP_F32 else 8
     CW = 4 if prec == L.LM_MLP_F32 else 8
+    parts = 2 if prec == L.LM_MLP_F16X2 else 1
+    _f = _frags
+    globals()["_frags"] = lambda *a: _f(*a, parts=parts)
     g = torch.Generator().manual_seed(1)
     ns = 37
     prod = torch.randn(ns, K, generator=g)
@@ -140,6 +161,7 @@ def test_packed_weights_replay_matches_oracle(lib, prec, dt, tol):
     h1 = np.maximum(_regs(_mma_layer(_frags(buf, lay["w1"], 4, 80, G, dt), s1)) + bias("b1", 4).transpose(1, 0, 2).reshape(2, 64), 0)
     h2 = np.maximum(_regs(_mma_layer(_frags(buf, lay["w2"], 4, 64, G, dt), h1)) + bias("b2", 4).transpose(1, 0, 2).reshape(2, 64), 0)
     o = _regs(_mma_layer(_frags(buf, lay["w3"], 1, 64, G, dt), h2)) + bias("b3", 1).transpose(1, 0, 2).reshape(2, 16)
+    globals()["_frags"] = _f
     rgb = 1 / (1 + np.exp(-o[:, 0, :3]))
     ref = O.mlp_render(p, view, torch.from_numpy(ref_feat)).numpy()
     assert np.allclose(rgb, ref, atol=tol)
