@@ -299,13 +299,14 @@ def main():
     ap.add_argument("--density-shift", type=float, default=0.0)
     ap.add_argument("--mlp", default="f16x2", choices=["f32", "f16x2", "f16", "bf16"])
     ap.add_argument("--term-eps", type=float, default=0.0)
-    ap.add_argument("--chunk", type=int, default=65536)
+    ap.add_argument("--chunk", type=int, default=262144)
     ap.add_argument("--queries", type=int, default=1 << 24)
     ap.add_argument("--rows", type=int, default=1 << 23)
     ap.add_argument("--coherent", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=8)
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calib", action="store_true", help="also run one 1 GiB device copy (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build renders on one GPU; rays are independent, so more GPUs would each take a slice of "
@@ -315,6 +316,12 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    if args.calib:
+        a = torch.ones(1 << 28, device="cuda:0")  # 1 GiB read + 1 GiB written by one copy kernel
+        b = torch.empty_like(a)
+        b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     if args.workload == "c2":
         out = bench_gather(args)
     elif args.workload == "c3":

@@ -216,7 +216,7 @@ int lm_app_products(const lm_model *model, const float *rays, const uint32_t *ap
                     float *products, void *stream);
 /* appearance samples (list order) -> feat [n_app,27] = basis_mat(plane*line products): the
  * gather fused with the projection, GridNeRF.compute_appfeature (gridnerf_sequential.py:829-871).
- * Needs equal channel counts per plane, a multiple of 16 (8 with LM_MLP_F32). */
+ * Needs a 16-bit matrix mode (not LM_MLP_F32) and equal channel counts per plane of 16, 32, 48 or 64. */
 int lm_app_features(const lm_model *model, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
                     float *feat, void *stream);
 

@@ -12,6 +12,8 @@
 // ((c+1)/2)*(size-1), corners floor/floor+1, out-of-range corners contribute zero.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
+
 #include "lm_common.h"
 #include "lm_mma.h"
 
@@ -272,82 +274,95 @@ template <> struct ChLoad<__half, 4> {
     }
 };
 
-template <int PREC, typename T, int NU>  // NU = groups of 2*CW channels per plane
-__global__ __launch_bounds__(256) void k_app_feat(lm_geom g, PlaneSet ps, int K, const char *__restrict__ packed,
-                                                  lm_mma::PackLayout L, const float *__restrict__ rays,
-                                                  const uint32_t *__restrict__ list,
-                                                  const uint32_t *__restrict__ count, float *__restrict__ feat) {
+template <int PREC> struct AppFeatBlock { static constexpr int N = 512; };
+
+// LDS: [basis fragments | one product tile per wave].  A tile is 32 samples x (C + 4) floats.
+__host__ __device__ inline size_t app_feat_tile_bytes(int C) { return (size_t)32 * (C + 4) * sizeof(float); }
+
+template <int PREC, typename T, int NU>  // NU = groups of 16 channels per plane (C = 16 * NU)
+__global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, PlaneSet ps, int K,
+                                                                   const char *__restrict__ packed, lm_mma::PackLayout L,
+                                                                   const float *__restrict__ rays,
+                                                                   const uint32_t *__restrict__ list,
+                                                                   const uint32_t *__restrict__ count,
+                                                                   float *__restrict__ feat) {
     using namespace lm_mma;
     using Mm = Mma<PREC>;
     using frag = typename Mm::frag;
-    constexpr int G = Mm::G, CW = Mm::CW, NP = Mm::NP;
+    constexpr int NP = Mm::NP;
+    constexpr int V = Vec<T>::V;
+    constexpr int C = 16 * NU, ROW = C + 4;
+    static_assert(Mm::G == 8 && Mm::CW == 8, "the fused gather feeds 16-bit MFMAs");
     extern __shared__ __align__(16) char lds[];
+    const size_t basis_bytes = (size_t)32 * K * sizeof(typename Mm::elem) * NP;
     {
-        const size_t bytes = (size_t)32 * K * sizeof(typename Mm::elem) * NP;
         const uint4 *src = reinterpret_cast<const uint4 *>(packed + L.basis);
         uint4 *dst = reinterpret_cast<uint4 *>(lds);
-        for (size_t i = threadIdx.x; i < bytes / 16; i += blockDim.x) dst[i] = src[i];
+        for (size_t i = threadIdx.x; i < basis_bytes / 16; i += blockDim.x) dst[i] = src[i];
         __syncthreads();
     }
     const frag *A = reinterpret_cast<const frag *>(lds);
     const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
+    const unsigned qlane = lane & 3u, gs = lane >> 2;  // gather role: 4 lanes per sample, 16 samples per pass
+    float *tile = reinterpret_cast<float *>(lds + basis_bytes + (threadIdx.x / LM_WAVE) * app_feat_tile_bytes(C));
     const uint64_t M = *count;
     const uint64_t n_tiles = (M + 31) / 32;
-    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * 4 + threadIdx.x / LM_WAVE;
-    const uint64_t n_waves = (uint64_t)gridDim.x * 4;
-    for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
-        const uint64_t p = tile * 32 + j;
-        const bool live = p < M;
-        float q[3];
-        list_coords(g, rays, list[live ? p : M - 1], q);
+    constexpr unsigned kWaves = AppFeatBlock<PREC>::N / LM_WAVE;
+    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * kWaves + threadIdx.x / LM_WAVE;
+    const uint64_t n_waves = (uint64_t)gridDim.x * kWaves;
+    for (uint64_t tile_id = wave_id; tile_id < n_tiles; tile_id += n_waves) {
+        // the two samples this lane gathers for (pass 0: tile row gs, pass 1: row 16 + gs)
+        float q0[3], q1[3];
+        {
+            const uint64_t p0 = tile_id * 32 + gs, p1 = p0 + 16;
+            list_coords(g, rays, list[p0 < M ? p0 : M - 1], q0);
+            list_coords(g, rays, list[p1 < M ? p1 : M - 1], q1);
+        }
         floatx16 acc;
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-        int t = 0;  // running MFMA step = slot / G over the concatenated channels
+        int t = 0;  // running MFMA step over the concatenated channels
         for (int k = 0; k < ps.n; ++k) {
             const lm_plane &pl = ps.p[k];
-            const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-            const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
-            const T *P = reinterpret_cast<const T *>(pl.plane);
-            const T *Ln = reinterpret_cast<const T *>(pl.line);
-            float a[NU][CW], b[NU][CW], c[NU][CW], d[NU][CW], l0[NU][CW], l1[NU][CW];
 #pragma unroll
-            for (int u = 0; u < NU; ++u) {
-                const int ch = 2 * CW * u + CW * (int)h;
-                ChLoad<T, CW>::load(P + t2.o00 + ch, a[u]);
-                ChLoad<T, CW>::load(P + t2.o01 + ch, b[u]);
-                ChLoad<T, CW>::load(P + t2.o10 + ch, c[u]);
-                ChLoad<T, CW>::load(P + t2.o11 + ch, d[u]);
-                ChLoad<T, CW>::load(Ln + t1.o0 + ch, l0[u]);
-                ChLoad<T, CW>::load(Ln + t1.o1 + ch, l1[u]);
-            }
+            for (int pass = 0; pass < 2; ++pass) {
+                const float *q = pass ? q1 : q0;
+                const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+                const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+                float *row = tile + (pass * 16 + gs) * ROW;
 #pragma unroll
-            for (int u = 0; u < NU; ++u) {
-                float prod[CW];
+                for (int c = V * (int)qlane; c < C; c += V * kQuad) {
+                    float prod[V];
+                    plane_products<T>(pl, t2, t1, c, prod);
 #pragma unroll
-                for (int i = 0; i < CW; ++i) {
-                    float pv = a[u][i] * t2.w00;
-                    pv = fmaf(b[u][i], t2.w01, pv);
-                    pv = fmaf(c[u][i], t2.w10, pv);
-                    pv = fmaf(d[u][i], t2.w11, pv);
-                    const float lv = fmaf(l1[u][i], t1.w1, l0[u][i] * t1.w0);
-                    prod[i] = pv * lv;
-                }
-#pragma unroll
-                for (int s = 0; s < CW / G; ++s, ++t) {
-                    frag bf[NP];
-                    Mm::pack(prod + s * G, bf);
-                    const frag a0 = A[(t * NP) * 64 + lane];
-                    acc = Mm::mma(a0, bf[0], acc);
-                    if constexpr (NP == 2) {
-                        const frag a1 = A[(t * NP + 1) * 64 + lane];
-                        acc = Mm::mma(a1, bf[0], acc);
-                        acc = Mm::mma(a0, bf[1], acc);
-                    }
+                    for (int i = 0; i < V; i += 4)
+                        *reinterpret_cast<float4 *>(row + c + i) = make_float4(prod[i], prod[i + 1], prod[i + 2], prod[i + 3]);
                 }
             }
+            // LDS operations of one wave complete in order; the fence only pins the compiler
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int u = 0; u < NU; ++u, ++t) {
+                const float4 *src = reinterpret_cast<const float4 *>(tile + j * ROW + 16 * u + 8 * (int)h);
+                const float4 x0 = src[0], x1 = src[1];
+                const float c8[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                frag bf[NP];
+                Mm::pack(c8, bf);
+                const frag a0 = A[(t * NP) * 64 + lane];
+                acc = Mm::mma(a0, bf[0], acc);
+                if constexpr (NP == 2) {
+                    const frag a1 = A[(t * NP + 1) * 64 + lane];
+                    acc = Mm::mma(a1, bf[0], acc);
+                    acc = Mm::mma(a0, bf[1], acc);
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
-        if (live) {
+        const uint64_t p = tile_id * 32 + j;
+        if (p < M) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int r = row_of(v, (int)h);
@@ -362,16 +377,19 @@ int launch_app_feat(int nu, const lm_model *m, const PlaneSet &ps, int K, const 
                     const uint32_t *count, float *feat, hipStream_t st) {
     using namespace lm_mma;
     const PackLayout L = pack_layout(PREC, K);
-    const size_t lds = (size_t)32 * K * sizeof(typename Mma<PREC>::elem) * Mma<PREC>::NP;
-    if (lds > 150 * 1024) LM_FAIL(LM_ERR_UNSUPPORTED, "basis_mat fragments (%zu bytes) do not fit LDS", lds);
-    const unsigned grid = (unsigned)lm_persistent_blocks(lds > 72 * 1024 ? 1 : 2);
+    constexpr int kThreads = AppFeatBlock<PREC>::N;
+    const size_t basis = (size_t)32 * K * sizeof(typename Mma<PREC>::elem) * Mma<PREC>::NP;
+    const size_t lds = basis + (kThreads / LM_WAVE) * app_feat_tile_bytes(16 * nu);
+    if (lds > 160 * 1024) LM_FAIL(LM_ERR_UNSUPPORTED, "basis_mat fragments + tiles (%zu bytes) do not fit LDS", lds);
+    const unsigned per_cu = (unsigned)std::max<size_t>(1, std::min<size_t>(2, (size_t)(160 * 1024) / lds));
+    const unsigned grid = (unsigned)lm_persistent_blocks((int)per_cu);
 #define LM_AF_CASE(NU_)                                                                                            \
     case NU_: {                                                                                                    \
         auto kern = &k_app_feat<PREC, T, NU_>;                                                                     \
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                  \
         if (e != hipSuccess) LM_FAIL(LM_ERR_LAUNCH, "k_app_feat: LDS reservation failed: %s", hipGetErrorString(e)); \
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, m->geom, ps, K, (const char *)m->mlp_packed, L, rays, \
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, st, m->geom, ps, K, (const char *)m->mlp_packed, L, rays, \
                            list, count, feat);                                                                     \
         break;                                                                                                     \
     }
@@ -497,13 +515,11 @@ extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint3
 
 // True when the fused gather + basis_mat kernel covers this model's appearance planes.
 int lm_app_feat_supported(const lm_model *m) {
-    const int cw = m->mlp_prec == LM_MLP_F32 ? 4 : 8;
+    if (m->mlp_prec == LM_MLP_F32) return 0;  // fp32 MFMAs take the unfused path
     const int C = m->app[0].C;
     for (int k = 0; k < m->n_planes; ++k)
         if (m->app[k].C != C) return 0;
-    if (C % (2 * cw) != 0) return 0;
-    const int nu = C / (2 * cw);
-    return nu >= 1 && nu <= 4;
+    return C % 16 == 0 && C >= 16 && C <= 64;
 }
 
 int lm_check_prec(int prec);
@@ -521,18 +537,15 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
     LM_REQUIRE(rays && app_idx && counters && feat, "null buffer");
     LM_REQUIRE(m->mlp_packed && lm_aligned16(m->mlp_packed), "packed colour-network weights are null or misaligned");
     if (!lm_app_feat_supported(m))
-        LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs equal channel counts, a multiple of %d",
-                m->mlp_prec == LM_MLP_F32 ? 8 : 16);
+        LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs a 16-bit matrix mode and equal channel counts of 16..64 in steps of 16");
     const PlaneSet ps = make_set(m->app, m->n_planes);
-    const int cw = m->mlp_prec == LM_MLP_F32 ? 4 : 8;
-    const int nu = m->app[0].C / (2 * cw);
+    const int nu = m->app[0].C / 16;
     hipStream_t st = (hipStream_t)stream;
     const uint32_t *cnt = counters + LM_STAT_N_APP;
 #define LM_AF_GO(PREC_)                                                                                    \
     return dtype == LM_F32 ? launch_app_feat<PREC_, float>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
                            : launch_app_feat<PREC_, __half>(nu, m, ps, K, rays, app_idx, cnt, feat, st)
     switch (m->mlp_prec) {
-        case LM_MLP_F32: LM_AF_GO(LM_MLP_F32);
         case LM_MLP_F16: LM_AF_GO(LM_MLP_F16);
         case LM_MLP_BF16: LM_AF_GO(LM_MLP_BF16);
         default: LM_AF_GO(LM_MLP_F16X2);
