@@ -10,7 +10,7 @@ times measured with HIP events inside the timed region, the roofline figure of t
 dominant kernel, and the CPU oracle timed on this box's host cores on a bounded sample
 of the same workload.
 
-Default workload: BASELINE config 4, a full 1920x1080 frame of a multi-resolution GridNeRF
+Default workload (the fourth benchmark configuration): a full 1920x1080 frame of a multi-resolution GridNeRF
 (levels 1024^2/2048^2/4096^2, 16 + 48 channels fp32, 256^3 occupancy at ~30 %, 128
 samples per ray).  The density shift is 0 so that every stage does work (with the stated
 N(0, 0.1) init and shift -10 every weight stays below the 1e-3 threshold and the colour
@@ -32,6 +32,13 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0, "bf16": 2500.0, "f16x2": 2500.0}
 MLP_FLOP_PER_ROW = 2 * (150 * 128 + 128 * 128 + 128 * 3)
+# HBM-side bytes per launch (L2 misses: FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs, scaled
+# by the factors a plain copy of known size gave: 2.00 and 1.00) of the default workload's gather
+# kernels at the default chunk size; any other configuration reports null.
+MEASURED_TRAFFIC = {
+    ("c4_1080p_multires_P3_base1024_shift0", 262144, "k_app_feat"): 4.17e9 + 0.10e9,
+    ("c4_1080p_multires_P3_base1024_shift0", 262144, "k_density_list"): 4.93e9 + 0.01e9,
+}
 
 
 def log(*a):
@@ -139,6 +146,7 @@ def bench_frame(args, workload):
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
     roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
     roof["launches_per_frame"] = launches
+    roof["traffic"] = MEASURED_TRAFFIC.get((name, chunk, roof["kernel"]))
 
     cpu, parity = cpu_baseline_frame(args, p, rays, rgb, depth, H, W)
     mrays = N / (ms_step * 1e-3) / 1e6
@@ -184,7 +192,7 @@ def cpu_baseline_frame(args, p, rays, rgb, depth, H, W):
 
 # ----------------------------------------------------------------------------------------
 def bench_gather(args):
-    """BASELINE config 2: isolated plane/line gather, 3 planes 2048^2 x 64 ch fp32, 2^24 queries."""
+    """Second benchmark configuration: isolated plane/line gather, 3 planes 2048^2 x 64 ch fp32, 2^24 queries."""
     from landmark_amd import scenes
     from landmark_amd.model import GridNeRFHIP
 
@@ -237,7 +245,7 @@ def bench_gather(args):
 
 
 def bench_mlp(args):
-    """BASELINE config 3: isolated colour network on 2^23 rows."""
+    """Third benchmark configuration: isolated colour network on 2^23 rows."""
     from landmark_amd import scenes
     from landmark_amd.model import GridNeRFHIP
 

@@ -1,6 +1,6 @@
 """GPU parity tests: the HIP path through the C-ABI against the CPU oracle.
 
-Bars (BASELINE north star): sample masks, sample counts and valid-sample indices
+Bars: sample masks, sample counts and valid-sample indices
 bit-exact; depths of the samples bit-exact; rgb / depth within 1e-4 absolute with fp32
 tables and an fp32 colour network, 1e-2 with fp16 tables or a 16-bit colour network.
 The appearance mask (weight > 1e-3) derives from floats that are summed in a different
@@ -237,7 +237,7 @@ def test_render_random_scenes(gpu_lib, opt, act, shift, res, ndims):
 
 
 def test_render_c1_tiny_config(gpu_lib):
-    """BASELINE config 1 at reduced image size (the oracle finishes in seconds): the stated
+    """The tiny full-render configuration at reduced image size (the oracle finishes in seconds): the stated
     init (background only) and the dense variant that runs every stage."""
     rays = scenes.c1_rays(64, 64)
     for dense in (False, True):
