@@ -39,7 +39,7 @@ typedef enum lm_status {
     LM_ERR_WORKSPACE = -4    /* workspace too small */
 } lm_status;
 
-enum { LM_F32 = 0, LM_F16 = 1 };                   /* plane / line storage type */
+enum { LM_F32 = 0, LM_F16 = 1, LM_U8 = 2, LM_CELLS = 3 }; /* planes: F32 | F16; occupancy: F32 | U8 | CELLS */
 enum { LM_SAMPLER_AABB = 0, LM_SAMPLER_HULL = 1 }; /* sampling_opt 0 / 1 */
 enum { LM_ACT_SOFTPLUS = 0, LM_ACT_RELU = 1 };     /* fea2denseAct */
 /* arithmetic of the colour network's and basis_mat's matrix products (accumulation is
@@ -79,8 +79,13 @@ typedef struct lm_geom {
     const float *tab_t; /* [S] */
     float inv_aabb[3];
     /* occupancy volume (app/models/alpha_mask.py); vol == NULL: no culling */
-    const float *vol; /* [vd][vh][vw] */
+    /* [vd][vh][vw] float, or uint8 (values a uint8 holds exactly), or the cell table
+     * lm_pack_occupancy builds from a 0/1 volume: [vd+1][vh+1][vw+1] bytes, one per trilinear
+     * cell, bit (zz*4 + yy*2 + xx) = voxel (z0+zz, y0+yy, x0+xx) is 1.  All three give
+     * bit-identical decisions; the cell table needs one load per sample instead of eight. */
+    const void *vol;
     int32_t vd, vh, vw;
+    int32_t vol_dtype; /* LM_F32 | LM_U8 | LM_CELLS */
     float vol_aabb_min[3];
     float vol_inv[3];
     float vol_thre; /* alpha_mask_filter_thre */
@@ -127,6 +132,13 @@ const char *lm_last_error(void);
  * out channel-last the same way (app/models/gridnerf_elastic_cuda.py:274-303). */
 int lm_relayout_nchw_to_hwc(const void *src, void *dst, int32_t C, int32_t H, int32_t W, int32_t dtype,
                             void *stream);
+
+/* Build the cell table of a 0/1 occupancy volume (float [D][H][W]); *not_binary (device
+ * uint32, zeroed by the caller) is set to 1 if a voxel is neither 0 nor 1, in which case the
+ * table must not be used.  cells: (D+1)*(H+1)*(W+1) bytes.  An internal acceleration
+ * structure for AlphaGridMask.sample_alpha (app/models/alpha_mask.py:35-47). */
+int lm_pack_occupancy(const float *vol, int32_t D, int32_t H, int32_t W, uint8_t *cells, uint32_t *not_binary,
+                      void *stream);
 
 /* ---- part 1: sampling + AABB / occupancy culling + stable compaction -----------------
  * Replaces sample_ray / sample_ray_within_hull + AlphaGridMask.sample_alpha + the

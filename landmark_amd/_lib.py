@@ -15,7 +15,7 @@ LM_MAX_PLANES = 12
 LM_N_STAGES = 6
 STAGE_NAMES = ["cull", "density", "weights", "app_gather", "colour", "composite"]
 LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_WORDS = 0, 1, 8
-LM_F32, LM_F16 = 0, 1
+LM_F32, LM_F16, LM_U8, LM_CELLS = 0, 1, 2, 3
 LM_SAMPLER_AABB, LM_SAMPLER_HULL = 0, 1
 LM_ACT_SOFTPLUS, LM_ACT_RELU = 0, 1
 LM_MLP_F32, LM_MLP_F16, LM_MLP_BF16, LM_MLP_F16X2 = 0, 1, 2, 3
@@ -34,7 +34,7 @@ class LmGeom(C.Structure):
     _fields_ = [
         ("sampler", C.c_int32), ("S", C.c_int32), ("aabb", C.c_float * 6), ("near_", C.c_float), ("far_", C.c_float),
         ("tab_a", C.c_void_p), ("tab_t", C.c_void_p), ("inv_aabb", C.c_float * 3),
-        ("vol", C.c_void_p), ("vd", C.c_int32), ("vh", C.c_int32), ("vw", C.c_int32),
+        ("vol", C.c_void_p), ("vd", C.c_int32), ("vh", C.c_int32), ("vw", C.c_int32), ("vol_dtype", C.c_int32),
         ("vol_aabb_min", C.c_float * 3), ("vol_inv", C.c_float * 3), ("vol_thre", C.c_float),
     ]
 
@@ -55,6 +55,7 @@ SYMBOLS = {
     "lm_abi_version": (C.c_int, []),
     "lm_last_error": (C.c_char_p, []),
     "lm_relayout_nchw_to_hwc": (C.c_int, [_P, _P, _I32, _I32, _I32, _I32, _P]),
+    "lm_pack_occupancy": (C.c_int, [_P, _I32, _I32, _I32, _P, _P, _P]),
     "lm_sample_cull_scratch_bytes": (_SZ, [_I64, _I32]),
     "lm_sample_cull": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "lm_gather_density_xyz": (C.c_int, [C.POINTER(LmPlane), _I32, _P, _I64, _P, _P]),

@@ -122,6 +122,17 @@ __device__ __forceinline__ float lm_alpha_lookup(const lm_geom &g, const float *
     fz = fminf(fmaxf(fz, -2.0f), (float)D);
     int x0 = (int)fx, y0 = (int)fy, z0 = (int)fz;
     float out = 0.0f;
+    if (g.vol_dtype == LM_CELLS) {
+        // one byte holds the eight corners of the cell (out-of-range corners are 0 bits); a set
+        // corner contributes 1.0f * w = w, added in the same order
+        if (x0 < -1 || x0 >= W || y0 < -1 || y0 >= H || z0 < -1 || z0 >= D) return 0.0f;
+        const size_t ci = ((size_t)(z0 + 1) * (H + 1) + (y0 + 1)) * (W + 1) + (x0 + 1);
+        const unsigned bits = reinterpret_cast<const uint8_t *>(g.vol)[ci];
+#pragma unroll
+        for (int n = 0; n < 8; ++n)
+            if (bits & (1u << n)) out = out + (wx[n & 1] * wy[(n >> 1) & 1]) * wz[n >> 2];
+        return out;
+    }
 #pragma unroll
     for (int zz = 0; zz < 2; ++zz)
 #pragma unroll
@@ -131,7 +142,10 @@ __device__ __forceinline__ float lm_alpha_lookup(const lm_geom &g, const float *
                 int x = x0 + xx, y = y0 + yy, z = z0 + zz;
                 if (x >= 0 && x < W && y >= 0 && y < H && z >= 0 && z < D) {
                     float w = (wx[xx] * wy[yy]) * wz[zz];
-                    float t = g.vol[((size_t)z * H + y) * W + x] * w;
+                    const size_t i = ((size_t)z * H + y) * W + x;
+                    const float val = g.vol_dtype == LM_U8 ? (float)reinterpret_cast<const uint8_t *>(g.vol)[i]
+                                                           : reinterpret_cast<const float *>(g.vol)[i];
+                    float t = val * w;
                     out = out + t;
                 }
             }

@@ -27,16 +27,25 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *
     for (int it = 0; it < kWordsPerWave; ++it) {
         const uint64_t w = w0 + it;
         if (w >= n_words) break;
-        const uint64_t flat = w * 64 + lane;
+        const uint32_t base = (uint32_t)(w * 64);  // total < 2^32 is checked by the caller
+        const uint32_t flat = base + lane;
         bool ok = false;
         if (flat < total) {
-            const uint64_t r = flat / (uint32_t)g.S;
-            const int s = (int)(flat - r * (uint32_t)g.S);
+            uint32_t r, s;
+            if (g.S % 64 == 0) {
+                // a wave never straddles two rays: ray index from wave-uniform values (scalar unit),
+                // and the ray's six floats come through scalar loads
+                r = (uint32_t)__builtin_amdgcn_readfirstlane((int)(base / (uint32_t)g.S));
+                s = base - r * (uint32_t)g.S + lane;
+            } else {
+                r = flat / (uint32_t)g.S;
+                s = flat - r * (uint32_t)g.S;
+            }
             float ray[6];
-            const float2 *rp = reinterpret_cast<const float2 *>(rays + 6 * r);
+            const float2 *rp = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
             float2 a = rp[0], b = rp[1], c = rp[2];
             ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
-            const float z = lm_sample_z(g, lm_ray_param(g, ray), s);
+            const float z = lm_sample_z(g, lm_ray_param(g, ray), (int)s);
             float pt[3];
             lm_point(ray, z, pt);
             ok = lm_sample_valid(g, pt);
@@ -113,6 +122,26 @@ __global__ __launch_bounds__(kBlock) void k_emit(const uint64_t *__restrict__ bi
     }
 }
 
+__global__ __launch_bounds__(256) void k_pack_occupancy(const float *__restrict__ vol, int D, int H, int W,
+                                                        uint8_t *__restrict__ cells, uint32_t *__restrict__ not_binary) {
+    const size_t n = (size_t)(D + 1) * (H + 1) * (W + 1);
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int cx = (int)(i % (W + 1)), cy = (int)((i / (W + 1)) % (H + 1)), cz = (int)(i / ((size_t)(W + 1) * (H + 1)));
+    unsigned bits = 0;
+    bool bad = false;
+    for (int k = 0; k < 8; ++k) {
+        const int x = cx - 1 + (k & 1), y = cy - 1 + ((k >> 1) & 1), z = cz - 1 + (k >> 2);
+        if (x >= 0 && x < W && y >= 0 && y < H && z >= 0 && z < D) {
+            const float v = vol[((size_t)z * H + y) * W + x];
+            if (v == 1.0f) bits |= 1u << k;
+            else if (v != 0.0f) bad = true;
+        }
+    }
+    cells[i] = (uint8_t)bits;
+    if (bad) *not_binary = 1u;  // plain store of the same value from every lane that sees one
+}
+
 }  // namespace
 
 static uint64_t n_blocks_for(uint64_t n_words) { return (n_words + kWordsPerBlock - 1) / kWordsPerBlock; }
@@ -128,7 +157,11 @@ int lm_check_geom(const lm_geom *g) {
     LM_REQUIRE(g->S > 0, "S must be positive (got %d)", g->S);
     LM_REQUIRE(g->sampler == LM_SAMPLER_AABB || g->sampler == LM_SAMPLER_HULL, "unknown sampler %d", g->sampler);
     LM_REQUIRE(g->tab_a && g->tab_t, "sampler tables are null");
-    if (g->vol) LM_REQUIRE(g->vd > 0 && g->vh > 0 && g->vw > 0, "occupancy volume has an empty dimension");
+    if (g->vol) {
+        LM_REQUIRE(g->vd > 0 && g->vh > 0 && g->vw > 0, "occupancy volume has an empty dimension");
+        LM_REQUIRE(g->vol_dtype == LM_F32 || g->vol_dtype == LM_U8 || g->vol_dtype == LM_CELLS,
+                   "occupancy volume dtype %d", g->vol_dtype);
+    }
     return LM_OK;
 }
 
@@ -164,5 +197,17 @@ extern "C" int lm_sample_cull(const lm_geom *geom, const float *rays, int64_t N,
     hipLaunchKernelGGL(k_emit, dim3((unsigned)nb), dim3(kBlock), 0, st, (const uint64_t *)bitmap, n_words,
                        (const uint32_t *)block_off, word_prefix, valid_idx);
     LM_CHECK_LAUNCH("k_emit");
+    return LM_OK;
+}
+
+extern "C" int lm_pack_occupancy(const float *vol, int32_t D, int32_t H, int32_t W, uint8_t *cells, uint32_t *not_binary,
+                                 void *stream) {
+    LM_REQUIRE(vol && cells && not_binary, "null buffer");
+    LM_REQUIRE(D > 0 && H > 0 && W > 0, "empty volume");
+    const size_t n = (size_t)(D + 1) * (H + 1) * (W + 1);
+    LM_REQUIRE(n < ((size_t)1 << 39), "volume too large");
+    hipLaunchKernelGGL(k_pack_occupancy, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, D, H, W,
+                       cells, not_binary);
+    LM_CHECK_LAUNCH("k_pack_occupancy");
     return LM_OK;
 }

@@ -45,6 +45,7 @@ class GridNeRFHIP:
         mlp_precision: str = "f32",
         term_eps: float = 0.0,
         release_source: bool = False,
+        occupancy: str = "auto",  # auto | cells | u8 | f32: storage of the occupancy volume
     ):
         if not torch.cuda.is_available():
             raise L.LandmarkError("GridNeRFHIP needs a GPU; there is no CPU path")
@@ -75,6 +76,19 @@ class GridNeRFHIP:
                 alpha_volume=vol.view(1, 1, *vol.shape[-3:]), aabb=params.alpha_aabb.to(self.device)
             )
         self._vol = None if self.alphaMask is None else self.alphaMask.alpha_volume
+        self._vol_dtype, self._vol_store = L.LM_F32, self._vol
+        if self._vol is not None and occupancy in ("auto", "cells", "u8"):
+            D, H, W = self._vol.shape[-3:]
+            cells = torch.empty((D + 1) * (H + 1) * (W + 1), dtype=torch.uint8, device=self.device)
+            flag = torch.zeros(1, dtype=torch.int32, device=self.device)
+            L.check(self.lib.lm_pack_occupancy(self._vol.data_ptr(), D, H, W, cells.data_ptr(), flag.data_ptr(), L.current_stream()), "lm_pack_occupancy")
+            if occupancy != "u8" and int(flag.item()) == 0:
+                # a 0/1 mask (what the reference stores): one byte per trilinear cell, one load per sample
+                self._vol_dtype, self._vol_store = L.LM_CELLS, cells
+            else:
+                as_u8 = self._vol.clamp(0, 255).to(torch.uint8)
+                if bool((as_u8.float() == self._vol).all()):
+                    self._vol_dtype, self._vol_store = L.LM_U8, as_u8.contiguous()
         # --- channel-last tables
         self._tables = []  # keep device tensors alive
         self._density = self._relayout_set(params.density_plane, params.density_line)
@@ -167,7 +181,8 @@ class GridNeRFHIP:
         g.tab_a, g.tab_t = a_d.data_ptr(), t_d.data_ptr()
         g.inv_aabb[:] = p.invaabbSize.detach().cpu().tolist()
         if self._vol is not None:
-            g.vol = self._vol.data_ptr()
+            g.vol = self._vol_store.data_ptr()
+            g.vol_dtype = self._vol_dtype
             g.vd, g.vh, g.vw = self._vol.shape[-3:]
             ab = p.alpha_aabb.detach().cpu()
             g.vol_aabb_min[:] = ab[0].tolist()

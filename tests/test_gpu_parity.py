@@ -62,6 +62,31 @@ def test_sample_cull_random_scene_bit_exact(gpu_lib, opt, S, thre):
     assert torch.equal(out["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
 
 
+@pytest.mark.parametrize("occupancy", ["f32", "u8", "cells"])
+def test_occupancy_storages_agree_bit_for_bit(gpu_lib, occupancy):
+    p = _scene(S=128, thre=0.5)
+    rays = scenes.pinhole_rays(96, 96, 80.0, scenes.sphere_pose(2.5, 5))
+    ref = O.render_chunk(p, rays, return_aux=True)
+    for thre in (0.0, 0.5, 0.98):
+        p.alpha_mask_filter_thre = thre
+        ref = O.render_chunk(p, rays, return_aux=True)
+        m = _model(p, occupancy=occupancy)
+        assert m._vol_dtype == {"f32": 0, "u8": 2, "cells": 3}[occupancy]
+        out = m.sample_cull(rays)
+        assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
+
+
+def test_non_binary_occupancy_falls_back_to_float(gpu_lib):
+    p = _scene(S=64, thre=0.2)
+    g = torch.Generator().manual_seed(3)
+    p.alpha_volume = torch.rand(p.alpha_volume.shape, generator=g)  # arbitrary float volume
+    rays = scenes.pinhole_rays(64, 64, 50.0, scenes.sphere_pose(2.5, 5))
+    ref = O.render_chunk(p, rays, return_aux=True)
+    m = _model(p)
+    assert m._vol_dtype == 0
+    assert torch.equal(m.sample_cull(rays)["ray_valid"].cpu(), ref["ray_valid"])
+
+
 def test_sample_cull_edge_cases(gpu_lib):
     p = _scene(with_mask=False, S=64)
     m = _model(p)
