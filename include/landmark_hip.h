@@ -4,7 +4,8 @@
  * entry point names the reference interface it replaces (paths relative to the
  * reference checkout).  Conventions:
  *   - plain pointers and sizes; all array pointers are DEVICE pointers unless the
- *     parameter is documented as host memory; device pointers must be 16-byte aligned;
+ *     parameter is documented as host memory; device pointers must be 16-byte aligned,
+ *     except ray arrays ([N,6] floats, any row of a 16-byte aligned array: 8-byte aligned);
  *   - the caller owns every buffer (inputs, outputs and the workspace); the library
  *     allocates nothing and keeps no global state besides a thread-local error string;
  *   - every function takes the HIP stream to launch on (`void*` = hipStream_t, NULL =

@@ -183,7 +183,8 @@ extern "C" int lm_sample_cull(const lm_geom *geom, const float *rays, int64_t N,
         return LM_OK;
     }
     LM_REQUIRE(rays && bitmap && word_prefix && valid_idx && scratch, "null buffer");
-    LM_REQUIRE(lm_aligned16(rays) && lm_aligned16(bitmap) && lm_aligned16(scratch), "buffers must be 16-byte aligned");
+    LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
+    LM_REQUIRE(lm_aligned16(bitmap) && lm_aligned16(scratch), "bitmap and scratch must be 16-byte aligned");
     const uint64_t n_words = (total + 63) / 64;
     const uint64_t nb = n_blocks_for(n_words);
     uint32_t *block_count = (uint32_t *)scratch;
