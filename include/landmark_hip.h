@@ -108,6 +108,10 @@ typedef struct lm_model {
     int32_t n_planes; /* ndims * levels, plane index k = dim * levels + level */
     lm_plane density[LM_MAX_PLANES];
     lm_plane app[LM_MAX_PLANES];
+    /* NULL, or basis_den.weight [n_planes * C_d] (device): density feature =
+     * relu(sum w * product) instead of the plain sum (nonlinear_density,
+     * gridnerf_sequential.py:679-680, 819-822) */
+    const float *density_basis;
     int32_t act;         /* LM_ACT_* */
     float density_shift; /* softplus(f + shift) */
     float distance_scale;
@@ -161,15 +165,16 @@ int lm_sample_cull(const lm_geom *geom, const float *rays, int64_t N, uint64_t *
 
 /* ---- part 2: plane / line feature gather ---------------------------------------------
  * Explicit normalised coordinates (isolated gather):
- *   lm_gather_density_xyz  out[M]        = sum_k sum_c plane_k,c(x) * line_k,c(x)
+ *   lm_gather_density_xyz  out[M]        = sum_k sum_c plane_k,c(x) * line_k,c(x), or with
+ *                          density_basis != NULL relu(sum_k sum_c w[k*C+c] * plane * line)
  *                          GridNeRF.compute_densityfeature, gridnerf_sequential.py:779-827;
  *                          prior art compute_appfeature.gridsample_sum_xyz_b
  *   lm_gather_app_xyz      out[M, n*C]   = plane_k,c(x) * line_k,c(x), column k*C + c
  *                          GridNeRF.compute_appfeature before basis_mat,
  *                          gridnerf_sequential.py:829-864; prior art gridsample_ew_xyb_bz
  */
-int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
-                          void *stream);
+int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, const float *density_basis, const float *xyz,
+                          int64_t M, float *out, void *stream);
 int lm_gather_app_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
                       void *stream);
 
@@ -184,6 +189,14 @@ int lm_gather_app_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz
 size_t lm_mlp_packed_bytes(int32_t prec, int32_t K_basis);
 int lm_mlp_pack(int32_t prec, int32_t K_basis, const float *basis, const float *w1, const float *b1,
                 const float *w2, const float *b2, const float *w3, const float *b3, void *packed_out);
+/* The appearance embedding (args.encode_app: MLPRender_Fea gets 48 more inputs between the
+ * features and the view direction, mlp_render_fea.py:23-24, 55-58) is constant over a frame,
+ * so its product with the first layer folds into that layer's bias: pack the layers with the
+ * 48 latent columns of W1 removed, and per frame write  b1 + W1[:, 27:75] @ embedding[app_code]
+ * into the packed buffer at lm_mlp_bias1_offset().  lm_mlp_pack_bias1: 128 host floats in
+ * natural order -> 128 host floats in the kernel's register order. */
+size_t lm_mlp_bias1_offset(int32_t prec, int32_t K_basis);
+int lm_mlp_pack_bias1(const float *b1, float *packed_b1_out);
 /* feat [M,27] fp32, view [M,3] fp32 -> rgb [M,3] fp32 */
 int lm_mlp(int32_t prec, const void *packed, int32_t K_basis, const float *feat, const float *view, int64_t M,
            float *rgb, void *stream);

@@ -43,7 +43,7 @@ class LmModel(C.Structure):
     _fields_ = [
         ("geom", LmGeom), ("n_planes", C.c_int32),
         ("density", LmPlane * LM_MAX_PLANES), ("app", LmPlane * LM_MAX_PLANES),
-        ("act", C.c_int32), ("density_shift", C.c_float), ("distance_scale", C.c_float), ("weight_thres", C.c_float),
+        ("density_basis", C.c_void_p), ("act", C.c_int32), ("density_shift", C.c_float), ("distance_scale", C.c_float), ("weight_thres", C.c_float),
         ("mlp_prec", C.c_int32), ("mlp_packed", C.c_void_p), ("white_bg", C.c_int32), ("term_eps", C.c_float),
         ("events", C.c_void_p * (LM_N_STAGES + 1)),
     ]
@@ -58,10 +58,12 @@ SYMBOLS = {
     "lm_pack_occupancy": (C.c_int, [_P, _I32, _I32, _I32, _P, _P, _P]),
     "lm_sample_cull_scratch_bytes": (_SZ, [_I64, _I32]),
     "lm_sample_cull": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _P, _P, _P, _P]),
-    "lm_gather_density_xyz": (C.c_int, [C.POINTER(LmPlane), _I32, _P, _I64, _P, _P]),
+    "lm_gather_density_xyz": (C.c_int, [C.POINTER(LmPlane), _I32, _P, _P, _I64, _P, _P]),
     "lm_gather_app_xyz": (C.c_int, [C.POINTER(LmPlane), _I32, _P, _I64, _P, _P]),
     "lm_mlp_packed_bytes": (_SZ, [_I32, _I32]),
     "lm_mlp_pack": (C.c_int, [_I32, _I32, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "lm_mlp_bias1_offset": (_SZ, [_I32, _I32]),
+    "lm_mlp_pack_bias1": (C.c_int, [_P, _P]),
     "lm_mlp": (C.c_int, [_I32, _P, _I32, _P, _P, _I64, _P, _P]),
     "lm_basis": (C.c_int, [_I32, _P, _I32, _P, _I64, _P, _P]),
     "lm_weights": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),

@@ -121,10 +121,14 @@ __device__ __forceinline__ void plane_products(const lm_plane &pl, const Taps2 &
     }
 }
 
+// den_w == NULL: plain sum over planes and channels.  Otherwise the reference's
+// nonlinear_density: relu(sum of den_w[plane*C + channel] * product) (gridnerf_sequential.py:819-822)
 template <typename T>
-__device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q, unsigned qlane) {
+__device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q, unsigned qlane,
+                                             const float *__restrict__ den_w) {
     constexpr int V = Vec<T>::V;
     float sum = 0.0f;
+    int col = 0;
     for (int k = 0; k < ps.n; ++k) {
         const lm_plane &pl = ps.p[k];
         const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
@@ -132,13 +136,19 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
         for (int c = V * qlane; c < pl.C; c += V * kQuad) {
             float prod[V];
             plane_products<T>(pl, t2, t1, c, prod);
+            if (den_w) {
 #pragma unroll
-            for (int i = 0; i < V; ++i) sum += prod[i];
+                for (int i = 0; i < V; ++i) sum = fmaf(den_w[col + c + i], prod[i], sum);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) sum += prod[i];
+            }
         }
+        col += pl.C;
     }
     sum += __shfl_xor(sum, 1);
     sum += __shfl_xor(sum, 2);
-    return sum;
+    return den_w ? fmaxf(sum, 0.0f) : sum;
 }
 
 template <typename T>
@@ -184,7 +194,8 @@ __device__ __forceinline__ float activate(float f, int act, float shift) {
 
 // ---- explicit coordinates ----------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float *__restrict__ xyz, uint64_t M,
+__global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float *__restrict__ den_w,
+                                                        const float *__restrict__ xyz, uint64_t M,
                                                         float *__restrict__ out) {
     const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
     const uint64_t n_tiles = (M + kTile - 1) / kTile;
@@ -192,7 +203,7 @@ __global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float
         const uint64_t p = tile * kTile + slot;
         if (p >= M) continue;
         float q[3] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2]};
-        const float s = density_sum<T>(ps, q, qlane);
+        const float s = density_sum<T>(ps, q, qlane, den_w);
         if (qlane == 0) out[p] = s;
     }
 }
@@ -212,7 +223,8 @@ __global__ __launch_bounds__(kBlock) void k_app_xyz(PlaneSet ps, int K, const fl
 
 // ---- list driven (inside the render) -------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps, const float *__restrict__ rays,
+__global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
+                                                         const float *__restrict__ rays,
                                                          const uint32_t *__restrict__ list,
                                                          const uint32_t *__restrict__ count, int act, float shift,
                                                          float *__restrict__ sigma) {
@@ -224,7 +236,7 @@ __global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps,
         if (p >= M) continue;
         float q[3];
         list_coords(g, rays, list[p], q);
-        const float s = density_sum<T>(ps, q, qlane);
+        const float s = density_sum<T>(ps, q, qlane, den_w);
         if (qlane == 0) sigma[p] = activate(s, act, shift);
     }
 }
@@ -436,8 +448,8 @@ static PlaneSet make_set(const lm_plane *planes, int n) {
     return ps;
 }
 
-extern "C" int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, const float *xyz, int64_t M, float *out,
-                                     void *stream) {
+extern "C" int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, const float *density_basis,
+                                     const float *xyz, int64_t M, float *out, void *stream) {
     int dtype;
     if (int rc = lm_check_planes(planes, n_planes, &dtype, nullptr)) return rc;
     LM_REQUIRE(M >= 0, "negative count");
@@ -447,9 +459,11 @@ extern "C" int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, c
     const uint64_t tiles = ((uint64_t)M + kTile - 1) / kTile;
     const unsigned grid = (unsigned)std::min<uint64_t>(tiles, (uint64_t)lm_persistent_blocks(8));
     if (dtype == LM_F32)
-        hipLaunchKernelGGL(k_density_xyz<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, xyz, (uint64_t)M, out);
+        hipLaunchKernelGGL(k_density_xyz<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, density_basis, xyz,
+                           (uint64_t)M, out);
     else
-        hipLaunchKernelGGL(k_density_xyz<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, xyz, (uint64_t)M, out);
+        hipLaunchKernelGGL(k_density_xyz<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, density_basis, xyz,
+                           (uint64_t)M, out);
     LM_CHECK_LAUNCH("k_density_xyz");
     return LM_OK;
 }
@@ -485,11 +499,11 @@ extern "C" int lm_density_valid(const lm_model *m, const float *rays, const uint
     const PlaneSet ps = make_set(m->density, m->n_planes);
     const unsigned grid = (unsigned)lm_persistent_blocks(8);
     if (dtype == LM_F32)
-        hipLaunchKernelGGL(k_density_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, rays,
-                           valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
+        hipLaunchKernelGGL(k_density_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps,
+                           m->density_basis, rays, valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
     else
-        hipLaunchKernelGGL(k_density_list<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, rays,
-                           valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
+        hipLaunchKernelGGL(k_density_list<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps,
+                           m->density_basis, rays, valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
     LM_CHECK_LAUNCH("k_density_list");
     return LM_OK;
 }

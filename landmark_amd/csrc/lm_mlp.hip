@@ -463,6 +463,19 @@ extern "C" int lm_mlp_pack(int32_t prec, int32_t K, const float *basis, const fl
     return LM_OK;
 }
 
+extern "C" size_t lm_mlp_bias1_offset(int32_t prec, int32_t K_basis) {
+    if (lm_check_prec(prec) || lm_check_K(K_basis)) return 0;
+    return pack_layout(prec, K_basis).b1;
+}
+
+extern "C" int lm_mlp_pack_bias1(const float *b1, float *packed_b1_out) {
+    LM_REQUIRE(b1 && packed_b1_out, "null pointer");
+    for (int fb = 0; fb < 4; ++fb)
+        for (int h = 0; h < 2; ++h)
+            for (int v = 0; v < 16; ++v) packed_b1_out[(fb * 2 + h) * 16 + v] = b1[32 * fb + row_of(v, h)];
+    return LM_OK;
+}
+
 static unsigned mlp_grid(uint64_t M) {
     const uint64_t tiles = (M + 31) / 32, wpb = 4, blocks = (tiles + wpb - 1) / wpb;
     return (unsigned)std::min<uint64_t>(std::max<uint64_t>(blocks, 1), (uint64_t)lm_persistent_blocks(1));

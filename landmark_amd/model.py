@@ -96,8 +96,23 @@ class GridNeRFHIP:
         self.K_app = sum(pl.C for pl in self._app)
         if release_source:
             params.density_plane, params.density_line, params.app_plane, params.app_line = [], [], [], []
-        # --- colour network
+        # --- density projection (nonlinear_density)
+        self._den_w = None
+        if params.nonlinear_density:
+            self._den_w = params.basis_den.detach().to(self.device, torch.float32).reshape(-1).contiguous()
+            if self._den_w.numel() != sum(pl.C for pl in self._density):
+                raise L.LandmarkError("basis_den width does not match the density planes")
+        # --- colour network; with encode_app the 48 latent columns of the first layer fold into its bias
+        self.encode_app = bool(params.encode_app)
+        self._latent_dim = 0
+        if self.encode_app:
+            self._latent_dim = params.embedding_app.shape[1]
+            self.embedding_app = params.embedding_app.detach().float().cpu()
+            w1 = params.mlp_w[0].detach().float().cpu()
+            self._w1_latent = w1[:, 27 : 27 + self._latent_dim].contiguous()  # [128, 48]
+            self._w1_plain = torch.cat([w1[:, :27], w1[:, 27 + self._latent_dim :]], 1).contiguous()  # [128, 150]
         self._packed = {}
+        self._bias_code = {}
         self._pack_mlp(mlp_precision)
         # --- per-S geometry and workspace caches
         self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
@@ -155,9 +170,12 @@ class GridNeRFHIP:
             keep.append(a)
             return a.ctypes.data
 
+        w1 = self._w1_plain if self.encode_app else p.mlp_w[0]
+        if tuple(w1.shape) != (128, 150):
+            raise L.LandmarkError(f"first colour layer has shape {tuple(w1.shape)}, expected (128, 150)")
         L.check(
             self.lib.lm_mlp_pack(
-                prec, K, f(p.basis_mat), f(p.mlp_w[0]), f(p.mlp_b[0]), f(p.mlp_w[1]), f(p.mlp_b[1]),
+                prec, K, f(p.basis_mat), f(w1), f(p.mlp_b[0]), f(p.mlp_w[1]), f(p.mlp_b[1]),
                 f(p.mlp_w[2]), f(p.mlp_b[2]), host.ctypes.data,
             ),
             "lm_mlp_pack",
@@ -165,6 +183,27 @@ class GridNeRFHIP:
         dev = torch.from_numpy(host).to(self.device)
         self._packed[precision] = (prec, dev)
         return self._packed[precision]
+
+    def _set_app_code(self, precision: str, app_code):
+        """Fold embedding_app[app_code] into the packed first-layer bias (512 bytes, stream ordered)."""
+        if not self.encode_app:
+            if app_code is not None:
+                raise NotImplementedError("app_code given but the model has no appearance embedding (encode_app)")
+            return
+        if app_code is None:
+            raise ValueError("this model was trained with encode_app: forward needs app_code")
+        code = int(app_code)
+        prec, packed = self._pack_mlp(precision)
+        if self._bias_code.get(precision) == code:
+            return
+        b1 = self.p.mlp_b[0]
+        b1 = torch.zeros(128) if b1 is None else b1.detach().float().cpu()
+        eff = (b1 + self._w1_latent @ self.embedding_app[code]).contiguous().numpy()
+        out = np.zeros(128, dtype=np.float32)
+        L.check(self.lib.lm_mlp_pack_bias1(eff.ctypes.data, out.ctypes.data), "lm_mlp_pack_bias1")
+        off = self.lib.lm_mlp_bias1_offset(prec, self.K_app)
+        packed[off : off + 512].copy_(torch.from_numpy(out.view(np.uint8)), non_blocking=False)
+        self._bias_code[precision] = code
 
     def _geom(self, S: int) -> L.LmGeom:
         if S in self._geom_cache:
@@ -198,6 +237,7 @@ class GridNeRFHIP:
         for k in range(len(self._density)):
             m.density[k] = self._density[k]
             m.app[k] = self._app[k]
+        m.density_basis = None if self._den_w is None else self._den_w.data_ptr()
         m.act = L.LM_ACT_SOFTPLUS if self.p.fea2denseAct == "softplus" else L.LM_ACT_RELU
         m.density_shift = self.p.density_shift
         m.distance_scale = self.p.distance_scale
@@ -237,8 +277,9 @@ class GridNeRFHIP:
         """GridBaseSequential.forward in render mode -> ({"rgb_map","depth_map"}, {})."""
         if is_train:
             raise NotImplementedError("training is outside this render path (is_train must be False)")
-        if app_code is not None or idxs_chunk is not None:
-            raise NotImplementedError("appearance embedding (encode_app) is not part of this render path")
+        if idxs_chunk is not None:
+            raise NotImplementedError("per-ray image indices (idxs_chunk) are a training input")
+        self._set_app_code(self.mlp_precision, app_code)
         rays = rays_chunk.to(self.device, torch.float32).contiguous()
         if rays.dim() != 2 or rays.shape[1] != 6:
             raise ValueError(f"rays_chunk must be [N,6], got {tuple(rays.shape)}")
@@ -320,7 +361,7 @@ class GridNeRFHIP:
         M = xyz.shape[0]
         out = torch.empty(M, dtype=torch.float32, device=self.device)
         arr = self._plane_array(self._density)
-        L.check(self.lib.lm_gather_density_xyz(arr, len(self._density), xyz.data_ptr(), M, out.data_ptr(), L.current_stream()), "lm_gather_density_xyz")
+        L.check(self.lib.lm_gather_density_xyz(arr, len(self._density), L.ptr(self._den_w), xyz.data_ptr(), M, out.data_ptr(), L.current_stream()), "lm_gather_density_xyz")
         return out
 
     @torch.no_grad()
@@ -348,8 +389,9 @@ class GridNeRFHIP:
         return self.basis(self.app_products(xyz_sampled), precision)
 
     @torch.no_grad()
-    def render_module(self, viewdirs, features, precision=None):
-        """MLPRender_Fea.forward(viewdirs, features) -> rgb [M,3]."""
+    def render_module(self, viewdirs, features, precision=None, app_code=None):
+        """MLPRender_Fea.forward(viewdirs, features[, latent of app_code]) -> rgb [M,3]."""
+        self._set_app_code(precision or self.mlp_precision, app_code)
         prec, packed = self._pack_mlp(precision or self.mlp_precision)
         feat = features.to(self.device, torch.float32).contiguous()
         view = viewdirs.to(self.device, torch.float32).contiguous()
@@ -458,5 +500,9 @@ def from_reference_model(model, **kw) -> GridNeRFHIP:
         alpha_volume=None if am is None else am.alpha_volume[0, 0].detach(),
         alpha_aabb=None if am is None else am.aabb.detach().cpu(),
         alpha_mask_filter_thre=float(model.alpha_mask_filter_thre),
+        encode_app=bool(getattr(model.args, "encode_app", False)),
+        embedding_app=model.embedding_app.weight.detach() if getattr(model.args, "encode_app", False) else None,
+        nonlinear_density=bool(getattr(model, "nonlinear_density", False)),
+        basis_den=model.basis_den.weight.detach() if getattr(model, "nonlinear_density", False) else None,
     )
     return GridNeRFHIP(p, **kw)

@@ -47,6 +47,13 @@ class GridNeRFParams:
     alpha_volume: Optional[torch.Tensor] = None  # [D,H,W] float {0,1}
     alpha_aabb: Optional[torch.Tensor] = None  # [2,3]
     alpha_mask_filter_thre: float = 0.0
+    # per-image appearance embedding (args.encode_app, gridnerf_sequential.py:681-682): the
+    # first Linear then takes 27 + 48 + 3 + 108 + 12 = 198 inputs (mlp_render_fea.py:23-24)
+    encode_app: bool = False
+    embedding_app: Optional[torch.Tensor] = None  # [n_images, 48]
+    # density through a learned projection (args.nonlinear_density, gridnerf_sequential.py:679-680, 819-822)
+    nonlinear_density: bool = False
+    basis_den: Optional[torch.Tensor] = None  # [1, P*L*C_d]
 
     # ---- derived quantities, gridnerf_sequential.py:149-164 -------------------------
     @property
@@ -103,4 +110,8 @@ class GridNeRFParams:
             alpha_volume=mv(self.alpha_volume),
             alpha_aabb=mv(self.alpha_aabb),
             alpha_mask_filter_thre=self.alpha_mask_filter_thre,
+            encode_app=self.encode_app,
+            embedding_app=mv(self.embedding_app),
+            nonlinear_density=self.nonlinear_density,
+            basis_den=mv(self.basis_den),
         )

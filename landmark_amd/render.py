@@ -12,8 +12,11 @@ from __future__ import annotations
 import torch
 
 
-def renderer_fn(rays, gridnerf, chunk=4096, N_samples=-1, white_bg=True, is_train=False, device="cuda", idxs=None):
-    """Returns ({"rgb_map": [N,3], "depth_map": [N]}, {})."""
+def renderer_fn(rays, gridnerf, chunk=4096, N_samples=-1, white_bg=True, is_train=False, device="cuda", idxs=None,
+                app_code=None):
+    """Returns ({"rgb_map": [N,3], "depth_map": [N]}, {}).  `app_code` (dist_render's
+    per-frame appearance code, inferer_impl.py:144-145) is forwarded when given."""
+    extra_kw = {} if app_code is None else {"app_code": app_code}
     all_ret = {}
     extra_loss = {}
     n_all = rays.shape[0]
@@ -23,7 +26,7 @@ def renderer_fn(rays, gridnerf, chunk=4096, N_samples=-1, white_bg=True, is_trai
             idxs_chunk = idxs[ci * chunk : (ci + 1) * chunk].to(device)
             ret, extra_loss = gridnerf(rays_chunk, is_train=is_train, white_bg=white_bg, N_samples=N_samples, idxs_chunk=idxs_chunk)
         else:
-            ret, extra_loss = gridnerf(rays_chunk, is_train=is_train, white_bg=white_bg, N_samples=N_samples)
+            ret, extra_loss = gridnerf(rays_chunk, is_train=is_train, white_bg=white_bg, N_samples=N_samples, **extra_kw)
         for k in ret:
             all_ret.setdefault(k, []).append(ret[k])
     all_ret = {k: torch.cat(v, 0) for k, v in all_ret.items()}

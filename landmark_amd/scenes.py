@@ -44,6 +44,9 @@ def make_params(
     dtype: torch.dtype = torch.float32,
     bias_enable: bool = True,
     feature_init: str = "normal",
+    encode_app: bool = False,
+    nonlinear_density: bool = False,
+    n_images: int = 16,
     **cfg,
 ) -> GridNeRFParams:
     """Random-init model.  On `device="cpu"` the global torch RNG is seeded and used
@@ -81,7 +84,12 @@ def make_params(
     fea_pe = cfg.pop("fea_pe", 2)
     featureC = cfg.pop("featureC", 128)
     basis, _ = _linear_init(app_dim, app_n_comp * ndims * len(resMode), bias=False)
-    in_c = mlp_in_dim(app_dim, view_pe, fea_pe)
+    basis_den = emb = None
+    if nonlinear_density:
+        basis_den, _ = _linear_init(1, density_n_comp * ndims * len(resMode), bias=False)
+    if encode_app:
+        emb = torch.randn(n_images, 48)  # torch.nn.Embedding default init
+    in_c = mlp_in_dim(app_dim, view_pe, fea_pe) + (48 if encode_app else 0)
     w1, b1 = _linear_init(featureC, in_c, bias_enable)
     w2, b2 = _linear_init(featureC, featureC, bias_enable)
     w3, b3 = _linear_init(3, featureC, bias_enable)
@@ -104,6 +112,10 @@ def make_params(
         view_pe=view_pe,
         fea_pe=fea_pe,
         featureC=featureC,
+        encode_app=encode_app,
+        embedding_app=mv(emb),
+        nonlinear_density=nonlinear_density,
+        basis_den=mv(basis_den),
         **cfg,
     )
 

@@ -114,16 +114,22 @@ def _f32(t):
 
 
 def density_feature(p, xyz):
-    """Sum over planes and channels of plane*line, gridnerf_sequential.py:790-827
-    (nonlinear_density=False, return_feat=False).  xyz is normalised [M,3]."""
+    """Sum over planes and channels of plane*line, or relu(basis_den(products)) when
+    nonlinear_density is set; gridnerf_sequential.py:790-827 (return_feat=False).
+    xyz is normalised [M,3]."""
     cp, cl = _coords(p, xyz)
     L = len(p.resMode)
     out = torch.zeros((xyz.shape[0],), device=xyz.device)
+    pcs, lcs = [], []
     for k in range(len(p.density_plane)):
         d = k // L
         pc = F.grid_sample(_f32(p.density_plane[k]), cp[[d]], align_corners=True).view(-1, xyz.shape[0])
         lc = F.grid_sample(_f32(p.density_line[k]), cl[[d]], align_corners=True).view(-1, xyz.shape[0])
+        pcs.append(pc)
+        lcs.append(lc)
         out = out + torch.sum(pc * lc, dim=0)
+    if getattr(p, "nonlinear_density", False):
+        out = F.relu(F.linear((torch.cat(pcs) * torch.cat(lcs)).T, p.basis_den))[..., 0]
     return out
 
 
@@ -176,10 +182,10 @@ def positional_encoding(x, freqs):
     return torch.cat([torch.sin(q), torch.cos(q)], dim=-1)
 
 
-def mlp_input(p, viewdirs, feats):
-    """Row layout of the network input, app/models/mlp_render_fea.py:55-65
-    (encode_app off): [feat | view | PE(feat) | PE(view)]."""
-    parts = [feats]
+def mlp_input(p, viewdirs, feats, latent=None):
+    """Row layout of the network input, app/models/mlp_render_fea.py:55-65:
+    [feat | latent (encode_app) | view | PE(feat) | PE(view)]."""
+    parts = [feats, latent] if (getattr(p, "encode_app", False) and latent is not None) else [feats]
     if p.view_pe > -1:
         parts.append(viewdirs)
     if p.fea_pe > 0:
@@ -189,9 +195,9 @@ def mlp_input(p, viewdirs, feats):
     return torch.cat(parts, dim=-1)
 
 
-def mlp_render(p, viewdirs, feats):
+def mlp_render(p, viewdirs, feats, latent=None):
     """app/models/mlp_render_fea.py:30-41,66-68: Linear-ReLU-Linear-ReLU-Linear-sigmoid."""
-    h = mlp_input(p, viewdirs, feats)
+    h = mlp_input(p, viewdirs, feats, latent)
     h = F.relu(F.linear(h, p.mlp_w[0], p.mlp_b[0]))
     h = F.relu(F.linear(h, p.mlp_w[1], p.mlp_b[1]))
     h = F.linear(h, p.mlp_w[2], p.mlp_b[2])
@@ -202,7 +208,7 @@ def mlp_render(p, viewdirs, feats):
 # whole chunk
 # --------------------------------------------------------------------------------------
 @torch.no_grad()
-def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False):
+def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False, app_code=None):
     """GridBaseSequential.forward with is_train=False,
     app/models/gridnerf_sequential.py:448-504 (sampling_opt=0) and :523-576
     (sampling_opt=1); the two branches differ only in the sampler."""
@@ -232,7 +238,12 @@ def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False):
     app_mask = weight > p.rayMarch_weight_thres
     if app_mask.any():
         feats = app_feature(p, xyz[app_mask])
-        rgb[app_mask] = mlp_render(p, viewdirs[app_mask], feats)
+        latent = None
+        if getattr(p, "encode_app", False) and app_code is not None:
+            # compute_app_latent, gridnerf_sequential.py:429-437: one embedding row for every sample
+            idx = torch.ones(feats.shape[0], dtype=torch.long, device=feats.device) * torch.as_tensor(app_code).long()
+            latent = F.embedding(idx, p.embedding_app)
+        rgb[app_mask] = mlp_render(p, viewdirs[app_mask], feats, latent)
 
     acc = torch.sum(weight, -1)
     rgb_map = torch.sum(weight[..., None] * rgb, -2)
@@ -257,7 +268,7 @@ def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False):
 
 
 def renderer_fn(
-    rays, model, chunk=4096, N_samples=-1, white_bg=True, is_train=False, device="cpu", idxs=None
+    rays, model, chunk=4096, N_samples=-1, white_bg=True, is_train=False, device="cpu", idxs=None, app_code=None
 ) -> Tuple[Dict[str, torch.Tensor], dict]:
     """Chunk loop, app/tools/render_utils.py:15-63, driving `render_chunk` on `model`
     (a parameter object).  `is_train` and `idxs` are accepted and must be off."""
@@ -265,7 +276,7 @@ def renderer_fn(
     acc: Dict[str, list] = {}
     n = rays.shape[0]
     for i in range(n // chunk + int(n % chunk > 0)):
-        ret = render_chunk(model, rays[i * chunk : (i + 1) * chunk].to(device), white_bg=white_bg, N_samples=N_samples)
+        ret = render_chunk(model, rays[i * chunk : (i + 1) * chunk].to(device), white_bg=white_bg, N_samples=N_samples, app_code=app_code)
         for k, v in ret.items():
             acc.setdefault(k, []).append(v)
     return {k: torch.cat(v, 0) for k, v in acc.items()}, {}

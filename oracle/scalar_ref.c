@@ -203,6 +203,9 @@ typedef struct {
     int softplus;
     float density_shift, distance_scale, weight_thres;
     int white_bg;
+    const float *basis_den; /* NULL, or [n_planes*C_d]: density = relu(sum w*product) (gridnerf_sequential.py:819-822) */
+    const float *latent;    /* NULL, or the frame's appearance embedding row (gridnerf_sequential.py:429-437) */
+    int latent_dim;
 } lmref_model;
 
 static void pe(const float *x, int n, int F, float *sin_out, float *cos_out) {
@@ -224,7 +227,7 @@ static void linear(const float *w, const float *b, const float *x, int in, int o
 }
 
 int lmref_mlp_in_dim(const lmref_model *m) {
-    return m->app_dim + 3 + 2 * m->fea_pe * m->app_dim + 2 * m->view_pe * 3;
+    return m->app_dim + (m->latent ? m->latent_dim : 0) + 3 + 2 * m->fea_pe * m->app_dim + 2 * m->view_pe * 3;
 }
 
 /* rgb[3] of one sample from its app features and view direction */
@@ -232,6 +235,7 @@ void lmref_colour(const lmref_model *m, const float *feat, const float *view, fl
     float in[512], h1[512], h2[512], o[3];
     int n = 0, A = m->app_dim;
     memcpy(in + n, feat, sizeof(float) * A); n += A;
+    if (m->latent) { memcpy(in + n, m->latent, sizeof(float) * m->latent_dim); n += m->latent_dim; }
     memcpy(in + n, view, sizeof(float) * 3); n += 3;
     pe(feat, A, m->fea_pe, in + n, in + n + A * m->fea_pe); n += 2 * A * m->fea_pe;
     pe(view, 3, m->view_pe, in + n, in + n + 3 * m->view_pe); n += 2 * 3 * m->view_pe;
@@ -271,7 +275,15 @@ void lmref_render(const lmref_model *m, const float *rays, long N, float *rgb_ma
             if (ok) {
                 normalise(g, pt, q);
                 float f = 0.0f;
-                for (int k = 0; k < m->n_planes; ++k) f += lmref_plane_products(&m->density[k], q, NULL);
+                if (m->basis_den) {
+                    int Cd = m->density[0].C;
+                    for (int k = 0; k < m->n_planes; ++k) {
+                        lmref_plane_products(&m->density[k], q, prod);
+                        for (int c = 0; c < Cd; ++c) f += m->basis_den[k * Cd + c] * prod[c];
+                    }
+                    f = f > 0.0f ? f : 0.0f;
+                } else
+                    for (int k = 0; k < m->n_planes; ++k) f += lmref_plane_products(&m->density[k], q, NULL);
                 if (m->softplus) {
                     float x = f + m->density_shift;
                     sigma[s] = x > 20.0f ? x : log1pf(expf(x));

@@ -48,6 +48,7 @@ class Model(C.Structure):
         ("b2", C.POINTER(C.c_float)), ("w3", C.POINTER(C.c_float)), ("b3", C.POINTER(C.c_float)),
         ("softplus", C.c_int), ("density_shift", C.c_float), ("distance_scale", C.c_float),
         ("weight_thres", C.c_float), ("white_bg", C.c_int),
+        ("basis_den", C.POINTER(C.c_float)), ("latent", C.POINTER(C.c_float)), ("latent_dim", C.c_int),
     ]
 
 
@@ -85,7 +86,7 @@ def sampler_tables(p, S):
 class ScalarModel:
     """Keeps the numpy buffers alive behind a `Model` struct built from a parameter object."""
 
-    def __init__(self, p, N_samples=-1, white_bg=True):
+    def __init__(self, p, N_samples=-1, white_bg=True, app_code=None):
         self.keep = []
         if p.sampling_opt:
             S = p.n_importance
@@ -151,6 +152,11 @@ class ScalarModel:
         m.density_shift, m.distance_scale = p.density_shift, p.distance_scale
         m.weight_thres = p.rayMarch_weight_thres
         m.white_bg = int(white_bg)
+        if getattr(p, "nonlinear_density", False):
+            m.basis_den = f(p.basis_den.reshape(-1))
+        if getattr(p, "encode_app", False) and app_code is not None:
+            m.latent = f(p.embedding_app[int(app_code)])
+            m.latent_dim = p.embedding_app.shape[1]
         self.model = m
 
     def sample_cull(self, rays):

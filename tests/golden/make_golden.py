@@ -111,6 +111,8 @@ CASES = [
     dict(name="hull_relu_L3_P1", grid=[5, 6, 4], dn=16, an=48, act="relu", shift=-10.0, res=[1, 2, 4], ndims=1, opt=1, mask=False, thre=0.0, S=24, boost=20.0),
     dict(name="aabb_softplus_L1", grid=[6, 7, 5], dn=16, an=48, act="softplus", shift=-1.0, res=[1], ndims=3, opt=0, mask=True, thre=0.0, S=20, boost=10.0, sr=0.25),
     dict(name="aabb_relu_L2_nomask", grid=[4, 5, 6], dn=8, an=12, act="relu", shift=-10.0, res=[1, 2], ndims=2, opt=0, mask=False, thre=0.0, S=-1, boost=15.0, sr=0.5),
+    dict(name="hull_relu_encodeapp_nonlinear", grid=[6, 7, 5], dn=16, an=48, act="relu", shift=-10.0, res=[1, 2], ndims=1, opt=1, mask=True, thre=0.5, S=16, boost=6.0, encode_app=True, nonlinear=True, app_code=3),
+    dict(name="aabb_softplus_encodeapp", grid=[5, 5, 6], dn=16, an=16, act="softplus", shift=-0.5, res=[1], ndims=3, opt=0, mask=False, thre=0.0, S=18, boost=8.0, sr=0.3, encode_app=True, app_code=5),
     dict(name="hull_softplus_trivial", grid=[6, 7, 5], dn=16, an=48, act="softplus", shift=-10.0, res=[1], ndims=3, opt=1, mask=False, thre=0.0, S=16, boost=1.0),
 ]
 
@@ -129,7 +131,7 @@ def main():
         aabb = torch.tensor([[-1.0, -1.2, -0.8], [1.1, 1.0, 0.9]])
         args = _args(
             ndims=c["ndims"], resMode=c["res"], sampling_opt=c["opt"], n_importance=max(c["S"], 8),
-            alpha_mask_filter_thre=c["thre"],
+            alpha_mask_filter_thre=c["thre"], encode_app=bool(c.get("encode_app")), nonlinear_density=bool(c.get("nonlinear")),
         )
         model = GridNeRF(
             aabb, c["grid"], "cpu",
@@ -139,7 +141,14 @@ def main():
             fea2denseAct=c["act"], args=args, is_train=False,
         )
         model.eval()
+        app_code = None
+        if c.get("encode_app"):
+            # the reference allocates 11500 embedding rows; eight are enough for a fixture
+            model.embedding_app = torch.nn.Embedding(8, 48)
+            app_code = torch.tensor(c["app_code"])
         with torch.no_grad():
+            if c.get("nonlinear"):
+                model.basis_den.weight.abs_()  # keep relu(basis_den(.)) away from an all-zero density
             for t in model.density_plane:
                 t.mul_(c["boost"])
             if c["mask"]:
@@ -148,8 +157,8 @@ def main():
                 mask_aabb = aabb + torch.tensor([[0.05, -0.02, 0.0], [0.0, 0.03, -0.04]])
                 model.alphaMask = AlphaGridMask("cpu", mask_aabb, vol)
             rays = _camera_rays(7, (1.4, -1.1, 1.9), 11 + ci) if c["opt"] else _generic_rays(40, 11 + ci)
-            (out, extra) = model(rays, is_train=False, white_bg=True, N_samples=c["S"])
-            (out_black, _) = model(rays, is_train=False, white_bg=False, N_samples=c["S"])
+            (out, extra) = model(rays, app_code=app_code, is_train=False, white_bg=True, N_samples=c["S"])
+            (out_black, _) = model(rays, app_code=app_code, is_train=False, white_bg=False, N_samples=c["S"])
             # sub-function vectors on the same model
             if c["opt"]:
                 pts, _, z, inside = model.sample_ray_within_hull(rays[:, :3], rays[:, 3:6], is_train=False, N_samples=model.n_importance)
@@ -159,7 +168,10 @@ def main():
             dens = model.compute_densityfeature(q)
             appf = model.compute_appfeature(q)
             vd = rays[:, None, 3:6].expand(pts.shape).reshape(-1, 3)
-            rgb = model.renderModule(vd, appf)
+            latent = None
+            if app_code is not None:
+                latent = model.embedding_app(torch.ones(appf.shape[0], dtype=torch.long) * app_code.long())
+            rgb = model.renderModule(vd, appf, latent)
             sig = model.feature2density(dens)
             dists = torch.cat((z[:, 1:] - z[:, :-1], torch.zeros_like(z[:, :1])), dim=-1)
             alpha, weight, t_last = raw2alpha(sig.view(z.shape), dists * model.distance_scale)
@@ -182,7 +194,8 @@ def main():
             grid=c["grid"], ndims=c["ndims"], resMode=c["res"], sampling_opt=c["opt"], N_samples=c["S"],
             n_importance=int(model.n_importance), near_far=[0.4, 4.0], density_shift=c["shift"],
             fea2denseAct=c["act"], step_ratio=float(model.step_ratio), thre=c["thre"], nSamples=int(model.nSamples),
-            stepSize=float(model.stepSize),
+            stepSize=float(model.stepSize), encode_app=bool(c.get("encode_app")), nonlinear_density=bool(c.get("nonlinear")),
+            app_code=c.get("app_code"),
         )
         arrays = {k: (v.detach().cpu().numpy() if torch.is_tensor(v) else np.asarray(v)) for k, v in store.items()}
         arrays["cfg_json"] = np.frombuffer(__import__("json").dumps(cfg).encode(), dtype=np.uint8)

@@ -46,5 +46,9 @@ def load_golden(name):
         alpha_volume=data.get("alpha_volume"),
         alpha_aabb=data.get("alpha_aabb"),
         alpha_mask_filter_thre=cfg["thre"],
+        encode_app=cfg.get("encode_app", False),
+        embedding_app=sd.get("embedding_app.weight"),
+        nonlinear_density=cfg.get("nonlinear_density", False),
+        basis_den=sd.get("basis_den.weight"),
     )
     return p, data, cfg

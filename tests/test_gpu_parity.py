@@ -42,7 +42,7 @@ def _scene(seed=3, grid=(9, 11, 13), opt=1, S=64, with_mask=True, thre=0.0, shif
 @pytest.mark.parametrize("name", golden_names())
 def test_sample_cull_golden(gpu_lib, name):
     p, d, cfg = load_golden(name)
-    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], return_aux=True)
+    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], return_aux=True, app_code=cfg.get("app_code"))
     out = _model(p).sample_cull(d["rays"], N_samples=cfg["N_samples"])
     assert torch.equal(out["z_vals"].cpu(), ref["z_vals"])
     assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
@@ -246,10 +246,11 @@ def _check_render(p, rays, tol, S=-1, white_bg=True, **kw):
 @pytest.mark.parametrize("name", golden_names())
 def test_render_golden_vectors(gpu_lib, name):
     p, d, cfg = load_golden(name)
-    out, _ = _model(p)(d["rays"], white_bg=True, N_samples=cfg["N_samples"])
+    code = cfg.get("app_code")
+    out, _ = _model(p)(d["rays"], app_code=code, white_bg=True, N_samples=cfg["N_samples"])
     assert (out["rgb_map"].cpu() - d["rgb_map"]).abs().max().item() <= RGB_TOL_F32
     assert (out["depth_map"].cpu() - d["depth_map"]).abs().max().item() <= RGB_TOL_F32
-    out, _ = _model(p)(d["rays"], white_bg=False, N_samples=cfg["N_samples"])
+    out, _ = _model(p)(d["rays"], app_code=code, white_bg=False, N_samples=cfg["N_samples"])
     assert (out["rgb_map"].cpu() - d["rgb_map_black"]).abs().max().item() <= RGB_TOL_F32
 
 
@@ -259,6 +260,32 @@ def test_render_random_scenes(gpu_lib, opt, act, shift, res, ndims):
     rays = scenes.pinhole_rays(80, 80, 70.0, scenes.sphere_pose(2.5, 9))
     ref, _ = _check_render(p, rays, RGB_TOL_F32, S=128)
     assert ref["app_mask"].any(), "scene must exercise the colour network"
+
+
+def test_appearance_embedding_and_density_projection(gpu_lib):
+    """encode_app (latent folded into the first layer's bias, switched per call) and
+    nonlinear_density against the oracle."""
+    p = _scene(S=64, resMode=(1, 2), encode_app=True, nonlinear_density=True, fea2denseAct="relu", boost=3.0)
+    p.basis_den.abs_()
+    rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    m = _model(p)
+    outs = {}
+    for code in (0, 7, 0):  # switching back and forth must re-fold the bias
+        ref = O.render_chunk(p, rays, app_code=code, return_aux=True)
+        assert ref["app_mask"].any()
+        out, _ = m(rays, app_code=torch.tensor(code))
+        band = ((ref["weight"] - 1e-3).abs() < 2e-7).any(-1)
+        assert (out["rgb_map"].cpu() - ref["rgb_map"]).abs().max(-1).values[~band].max().item() <= RGB_TOL_F32
+        assert (out["depth_map"].cpu() - ref["depth_map"]).abs()[~band].max().item() <= RGB_TOL_F32
+        outs.setdefault(code, []).append(out["rgb_map"])
+    assert torch.equal(outs[0][0], outs[0][1]) and not torch.equal(outs[0][0], outs[7][0])
+    g = torch.Generator().manual_seed(1)
+    xyz = torch.rand(3000, 3, generator=g) * 2 - 1
+    assert torch.allclose(m.compute_densityfeature(xyz).cpu(), O.density_feature(p, xyz), atol=2e-5)
+    with pytest.raises(ValueError):
+        m(rays)  # a model with an embedding needs the code
+    with pytest.raises(NotImplementedError):
+        _model(_scene(S=64))(rays, app_code=1)
 
 
 def test_render_c1_tiny_config(gpu_lib):

@@ -51,9 +51,9 @@ def test_argument_validation_returns_status_not_abort(lib):
     assert lib.lm_mlp_packed_bytes(7, 144) == 0
     assert lib.lm_mlp_packed_bytes(L.LM_MLP_F32, 100) == 0  # K not a multiple of 16
     pl = (L.LmPlane * 1)()
-    rc = lib.lm_gather_density_xyz(pl, 1, None, 10, None, None)
+    rc = lib.lm_gather_density_xyz(pl, 1, None, None, 10, None, None)
     assert rc == -1 and b"null table" in lib.lm_last_error()
-    assert lib.lm_gather_density_xyz(pl, 13, None, 10, None, None) == -1
+    assert lib.lm_gather_density_xyz(pl, 13, None, None, 10, None, None) == -1
     assert lib.lm_relayout_nchw_to_hwc(None, None, 4, 4, 4, 0, None) == -1
 
 

@@ -17,10 +17,10 @@ def test_fixtures_present():
 @pytest.mark.parametrize("name", NAMES)
 def test_forward_matches_reference(name):
     p, d, cfg = load_golden(name)
-    out = O.render_chunk(p, d["rays"], white_bg=True, N_samples=cfg["N_samples"])
+    out = O.render_chunk(p, d["rays"], white_bg=True, N_samples=cfg["N_samples"], app_code=cfg.get("app_code"))
     assert torch.equal(out["rgb_map"], d["rgb_map"])
     assert torch.equal(out["depth_map"], d["depth_map"])
-    out_b = O.render_chunk(p, d["rays"], white_bg=False, N_samples=cfg["N_samples"])
+    out_b = O.render_chunk(p, d["rays"], white_bg=False, N_samples=cfg["N_samples"], app_code=cfg.get("app_code"))
     assert torch.equal(out_b["rgb_map"], d["rgb_map_black"])
 
 
@@ -41,7 +41,10 @@ def test_subfunctions_match_reference(name):
     feats = O.app_feature(p, q)
     assert torch.equal(feats, d["sub_app_feature"])
     vd = d["rays"][:, None, 3:6].expand(pts.shape).reshape(-1, 3)
-    assert torch.equal(O.mlp_render(p, vd, feats), d["sub_rgb"])
+    latent = None
+    if cfg.get("encode_app"):
+        latent = p.embedding_app[cfg["app_code"]][None].expand(feats.shape[0], 48)
+    assert torch.equal(O.mlp_render(p, vd, feats, latent), d["sub_rgb"])
     sig = O.feature2density(p, d["sub_density_feature"]).view(z.shape)
     dists = torch.cat((z[:, 1:] - z[:, :-1], torch.zeros_like(z[:, :1])), dim=-1)
     a, w, t = O.raw2alpha(sig, dists * p.distance_scale)

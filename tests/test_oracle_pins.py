@@ -19,8 +19,8 @@ from tests.helpers import golden_names, load_golden
 @pytest.mark.parametrize("name", golden_names())
 def test_scalar_restatement_matches_oracle(name):
     p, d, cfg = load_golden(name)
-    sm = SR.ScalarModel(p, N_samples=cfg["N_samples"])
-    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], return_aux=True)
+    sm = SR.ScalarModel(p, N_samples=cfg["N_samples"], app_code=cfg.get("app_code"))
+    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], return_aux=True, app_code=cfg.get("app_code"))
     valid, z, cnt = sm.sample_cull(d["rays"])
     assert torch.equal(z, ref["z_vals"]), "z values must be bit-identical"
     assert torch.equal(valid, ref["ray_valid"]), "sample mask must be bit-identical"
