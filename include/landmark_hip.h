@@ -235,6 +235,17 @@ size_t lm_render_workspace_bytes(const lm_model *model, int64_t N);
 int lm_render(const lm_model *model, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
               float *rgb_map, float *depth_map, uint32_t *counters, void *stream);
 
+/* ---- either side of the path in the serving loop ------------------------------------------
+ * lm_generate_rays: rays[j*W+i] = (pose[:,3], pose[:,:3] @ (dir_x[i], dir_y[j], -1)), the
+ * pinhole rays of dist_render/dataset/utils.py:57-113 (generate_rays).  dir_x [W] and dir_y [H]
+ * are the reference's two torch.arange tables (device memory; computed by the caller so they
+ * hold the reference's values), pose_3x4 is HOST memory, row-major.
+ * lm_rgba8: rgb [N,3] in [0,1] -> [N,4] bytes (r,g,b,255) with torch's truncating float->uint8
+ * conversion, the tail of model_infer_postprocess (dist_render/ddp_infer/nerf_inferer.py:366-370). */
+int lm_generate_rays(const float *dir_x, const float *dir_y, const float *pose_3x4, int32_t H, int32_t W, float *rays,
+                     void *stream);
+int lm_rgba8(const float *rgb, int64_t N, uint8_t *rgba, void *stream);
+
 /* Stage-level pieces of lm_render for validation and profiling (same kernels). */
 int lm_density_valid(const lm_model *model, const float *rays, const uint32_t *valid_idx,
                      const uint32_t *counters, float *sigma, void *stream);

@@ -70,6 +70,8 @@ SYMBOLS = {
     "lm_render_workspace_bytes": (_SZ, [C.POINTER(LmModel), _I64]),
     "lm_app_features": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
     "lm_render": (C.c_int, [C.POINTER(LmModel), _P, _I64, _P, _SZ, _P, _P, _P, _P]),
+    "lm_generate_rays": (C.c_int, [_P, _P, _P, _I32, _I32, _P, _P]),
+    "lm_rgba8": (C.c_int, [_P, _I64, _P, _P]),
     "lm_density_valid": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
     "lm_app_products": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
 }

@@ -14,7 +14,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SO_PATH = os.path.join(HERE, "liblandmark_hip.so")
-SOURCES = ["lm_api.hip", "lm_sample.hip", "lm_gather.hip", "lm_mlp.hip", "lm_composite.hip"]
+SOURCES = ["lm_api.hip", "lm_sample.hip", "lm_gather.hip", "lm_mlp.hip", "lm_composite.hip", "lm_frame.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fhip-fp32-correctly-rounded-divide-sqrt", "-fno-fast-math",

@@ -52,3 +52,41 @@ class MultiBlockParallelHIP:
         return ret
 
     __call__ = forward
+
+
+def ray_direction_tables(H, W, focal):
+    """The two torch.arange tables of get_ray_directions_blender_faster
+    (dist_render/dataset/utils.py:57-72), evaluated on the host."""
+    cx, cy = W / 2, H / 2
+    dx = torch.arange(-cx / focal, (W - cx - 1e-5) / focal, 1 / focal, dtype=torch.float32)
+    dy = torch.arange(cy / focal, (cy - H + 1e-5) / focal, -1 / focal, dtype=torch.float32)
+    if dx.numel() != W or dy.numel() != H:
+        raise ValueError(f"direction tables have {dx.numel()}x{dy.numel()} entries for a {W}x{H} image")
+    return dx, dy
+
+
+def generate_rays(single_pose, H, W, focal=None, device="cuda"):
+    """[H*W, 6] rays on the GPU from a [3,4+] pose; `focal` defaults to pose[-1,-1]
+    (generate_rays, dist_render/dataset/utils.py:92-113)."""
+    from . import _lib as L
+
+    pose = torch.as_tensor(single_pose, dtype=torch.float32).cpu()
+    if focal is None:
+        focal = float(pose[-1, -1])
+    dx, dy = ray_direction_tables(int(H), int(W), float(focal))
+    dx, dy = dx.to(device), dy.to(device)
+    p34 = pose[:3, :4].contiguous().numpy()
+    rays = torch.empty((int(H) * int(W), 6), dtype=torch.float32, device=device)
+    L.check(L.load().lm_generate_rays(dx.data_ptr(), dy.data_ptr(), p34.ctypes.data, int(H), int(W), rays.data_ptr(), L.current_stream()), "lm_generate_rays")
+    return rays
+
+
+def postprocess_rgba8(rgb_map, H, W):
+    """[H,W,4] uint8 image (alpha 255) from rgb in [0,1]
+    (model_infer_postprocess, dist_render/ddp_infer/nerf_inferer.py:366-370)."""
+    from . import _lib as L
+
+    rgb = rgb_map.contiguous()
+    out = torch.empty((int(H), int(W), 4), dtype=torch.uint8, device=rgb.device)
+    L.check(L.load().lm_rgba8(rgb.data_ptr(), rgb.shape[0], out.data_ptr(), L.current_stream()), "lm_rgba8")
+    return out

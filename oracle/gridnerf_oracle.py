@@ -292,3 +292,31 @@ def to_fp16_features(p):
     q.app_plane = [t.half() for t in p.app_plane]
     q.app_line = [t.half() for t in p.app_line]
     return q
+
+
+# --------------------------------------------------------------------------------------
+# either side of the path in the serving loop
+# --------------------------------------------------------------------------------------
+def generate_rays(single_pose, H, W, focal=None):
+    """dist_render/dataset/utils.py:57-113 on the CPU: two arange tables, z = -1,
+    directions @ pose[:3,:3].T, origin = pose[:3,3].  Pinned by its closed form
+    ((i - W/2)/f, -(j - H/2)/f, -1) rotated by the pose."""
+    pose = torch.as_tensor(single_pose, dtype=torch.float32)
+    if focal is None:
+        focal = float(pose[-1, -1])
+    cx, cy = W / 2, H / 2
+    d = torch.empty((3, H, W), dtype=torch.float32)
+    d[0] = torch.arange(-cx / focal, (W - cx - 1e-5) / focal, 1 / focal, dtype=torch.float32).view(1, W)
+    d[1] = torch.arange(cy / focal, (cy - H + 1e-5) / focal, -1 / focal, dtype=torch.float32).view(H, 1)
+    d[2] = -1
+    d = d.permute(1, 2, 0)
+    rays_d = d @ pose[:3, :3].T
+    rays_o = pose[:3, 3].expand(rays_d.shape)
+    return torch.cat([rays_o.reshape(-1, 3), rays_d.reshape(-1, 3)], 1)
+
+
+def postprocess_rgba8(rgb_map, H, W):
+    """dist_render/ddp_infer/nerf_inferer.py:366-370."""
+    r = rgb_map.reshape(H, W, 3) * 255
+    r = torch.cat([r, torch.ones((H, W, 1)) * 255], dim=-1)
+    return r.byte()

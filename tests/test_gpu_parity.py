@@ -336,3 +336,18 @@ def test_early_termination_bounds(gpu_lib):
     # background term (<= 1e-4); depth loses at most T * z_far
     assert (term["rgb_map"] - exact["rgb_map"]).abs().max().item() <= 1e-4
     assert (term["depth_map"] - exact["depth_map"]).abs().max().item() <= 1e-4 * 4.5 * 1.5
+
+
+def test_ray_generation_and_rgba8(gpu_lib):
+    from landmark_amd.render import generate_rays, postprocess_rgba8
+
+    pose = torch.cat([scenes.orbit_pose(2.6, 1.9, 7), torch.tensor([[0.0], [0.0], [1483.6378]])], 1)
+    for H, W in ((1080, 1920), (7, 5)):
+        got = generate_rays(pose, H, W).cpu()
+        ref = O.generate_rays(pose, H, W)
+        assert torch.equal(got[:, :3], ref[:, :3])
+        assert (got[:, 3:] - ref[:, 3:]).abs().max().item() <= 2e-7  # three-term dot product, order / fma differ
+    g = torch.Generator().manual_seed(0)
+    rgb = torch.rand(480 * 640, 3, generator=g)
+    rgb[:4] = torch.tensor([[0.0, 1.0, 0.5], [0.999, 0.0039, 0.00392157], [1.0, 1.0, 1.0], [0.0, 0.0, 0.0]])
+    assert torch.equal(postprocess_rgba8(rgb.cuda(), 480, 640).cpu(), O.postprocess_rgba8(rgb, 480, 640))

@@ -229,3 +229,18 @@ def test_normalize_coord_maps_corners():
     p = scenes.make_params(seed=0, aabb=((-3, -3, -0.1), (3, 3, 1)), gridSize=(4, 4, 4), density_n_comp=2, app_n_comp=2)
     assert torch.equal(O.normalize_coord(p, p.aabb[0][None]), -torch.ones(1, 3))
     assert torch.allclose(O.normalize_coord(p, p.aabb[1][None]), torch.ones(1, 3), atol=1e-6)
+
+
+def test_ray_generation_closed_form_and_rgba8():
+    pose = torch.cat([scenes.sphere_pose(2.5, 3), torch.tensor([[0.0], [0.0], [77.5]])], 1)  # focal in pose[-1,-1]
+    H, W = 9, 12
+    rays = O.generate_rays(pose, H, W)
+    assert rays.shape == (H * W, 6) and torch.equal(rays[:, :3], pose[:3, 3].expand(H * W, 3))
+    j, i = torch.meshgrid(torch.arange(H).float(), torch.arange(W).float(), indexing="ij")
+    dirs = torch.stack([(i - W / 2) / 77.5, -(j - H / 2) / 77.5, -torch.ones_like(i)], -1).reshape(-1, 3)
+    assert torch.allclose(rays[:, 3:], dirs @ pose[:3, :3].T, atol=1e-6)
+    # the same rays as the app-side generator (ray_utils.py:492-531)
+    assert torch.allclose(rays, scenes.pinhole_rays(H, W, 77.5, pose[:, :4]), atol=1e-6)
+    rgb = torch.tensor([[0.0, 1.0, 0.5], [0.999, 0.0039, 0.00392157]])
+    out = O.postprocess_rgba8(rgb, 1, 2)
+    assert out.dtype == torch.uint8 and out.tolist() == [[[0, 255, 127, 255], [254, 0, 1, 255]]]
