@@ -296,8 +296,8 @@ def bench_mlp(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--planes", type=int, default=3, help="ndims of the c4 model (3 = XY,XZ,YZ; 1 = XY only)")
     ap.add_argument("--base", type=int, default=1024, help="base plane resolution of c4 (levels x1,x2,x4)")

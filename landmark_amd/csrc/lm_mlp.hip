@@ -35,13 +35,23 @@
 #include "lm_common.h"
 #include "lm_mma.h"
 
+#ifndef LM_MLP16_THREADS
+#define LM_MLP16_THREADS 512
+#endif
+#ifndef LM_MLP_NCB
+#define LM_MLP_NCB 2
+#endif
+
 namespace {
 
 using namespace lm_mma;
 
 // 16-bit modes: 8 waves per workgroup (two per SIMD, 256 registers each); the split and fp32
 // modes need the full register file of a SIMD per wave
-template <int PREC> struct MlpBlock { static constexpr int N = (PREC == LM_MLP_F16 || PREC == LM_MLP_BF16) ? 512 : 256; };
+template <int PREC> struct MlpBlock {
+    static constexpr int N = (PREC == LM_MLP_F16 || PREC == LM_MLP_BF16) ? LM_MLP16_THREADS : 256;
+    static constexpr int NCB = PREC == LM_MLP_F32 ? 1 : LM_MLP_NCB;  // 32-sample column blocks per wave
+};
 
 // ---- host-side packing ----------------------------------------------------------------------
 // column of the reference's 150-wide input row that feeds slot (h, group, v); -1 = none
@@ -157,85 +167,90 @@ __device__ __forceinline__ void sincos_f32(float x, float &s, float &c) {
     c = ((q + 1) & 2) ? -cc : cc;
 }
 
-// One dense layer on the wave's 32 samples: acc[fb] (+)= W[32*fb .. +32, :] x B for NB row
-// blocks.  Steps run outermost so that the NB accumulator chains are independent and each
-// B fragment is used NB times; the weight fragments of step t+1 are fetched while step t
-// multiplies, and a scheduling barrier per step keeps the compiler from hoisting more.
-template <int PREC, int NB, int T>
+// One dense layer on the wave's 32*NCB samples: acc[fb][cb] (+)= W[32*fb .. +32, :] x B[cb]
+// for NB row blocks and NCB column blocks of 32 samples.  Every weight fragment read from
+// LDS feeds NCB MFMAs (an A fragment is 1 KB per 32-cycle MFMA, which is exactly the LDS
+// bandwidth of a CU when nothing is reused).  Steps run outermost so that the NB*NCB
+// accumulator chains are independent.  The fragments of step t+PF are requested while
+// step t multiplies; scheduling barriers keep the reads ahead of the MFMAs and stop the
+// compiler from hoisting every read to the top.
+template <int PREC, int NB, int NCB, int T, int PF>
 __device__ __forceinline__ void dense_layer(const typename Mma<PREC>::frag *W0, int fb0, unsigned lane,
-                                            const typename Mma<PREC>::frag (*b)[Mma<PREC>::NP], floatx16 *acc) {
-    const typename Mma<PREC>::frag *W = W0 + (size_t)fb0 * T * Mma<PREC>::NP * 64;
+                                            const typename Mma<PREC>::frag (*b)[T][Mma<PREC>::NP],
+                                            floatx16 (*acc)[NCB]) {
     using M = Mma<PREC>;
     using frag = typename M::frag;
     constexpr int NP = M::NP;
-    constexpr bool kPrefetch = NP == 1;  // the split mode has no registers to spare for a second buffer
-    frag cur[NB][NP], nxt[NB][NP];
+    const frag *W = W0 + (size_t)fb0 * T * NP * 64 + lane;
+    frag a[T][NB][NP];
 #pragma unroll
-    for (int fb = 0; fb < NB; ++fb)
+    for (int t = 0; t < PF && t < T; ++t)
 #pragma unroll
-        for (int pt = 0; pt < NP; ++pt) cur[fb][pt] = W[((fb * T + 0) * NP + pt) * 64 + lane];
+        for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+            for (int pt = 0; pt < NP; ++pt) a[t][fb][pt] = W[((fb * T + t) * NP + pt) * 64];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-        if (kPrefetch && t + 1 < T) {
+        if (t + PF < T) {
 #pragma unroll
             for (int fb = 0; fb < NB; ++fb)
 #pragma unroll
-                for (int pt = 0; pt < NP; ++pt) nxt[fb][pt] = W[((fb * T + t + 1) * NP + pt) * 64 + lane];
+                for (int pt = 0; pt < NP; ++pt) a[t + PF][fb][pt] = W[((fb * T + t + PF) * NP + pt) * 64];
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int fb = 0; fb < NB; ++fb) {
-            acc[fb] = M::mma(cur[fb][0], b[t][0], acc[fb]);
-            if constexpr (NP == 2) {
-                acc[fb] = M::mma(cur[fb][1], b[t][0], acc[fb]);
-                acc[fb] = M::mma(cur[fb][0], b[t][1], acc[fb]);
+        for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                acc[fb][cb] = M::mma(a[t][fb][0], b[cb][t][0], acc[fb][cb]);
+                if constexpr (NP == 2) {
+                    acc[fb][cb] = M::mma(a[t][fb][1], b[cb][t][0], acc[fb][cb]);
+                    acc[fb][cb] = M::mma(a[t][fb][0], b[cb][t][1], acc[fb][cb]);
+                }
             }
-        }
-        if (t + 1 < T) {
-#pragma unroll
-            for (int fb = 0; fb < NB; ++fb)
-#pragma unroll
-                for (int pt = 0; pt < NP; ++pt)
-                    cur[fb][pt] = kPrefetch ? nxt[fb][pt] : W[((fb * T + t + 1) * NP + pt) * 64 + lane];
-        }
         __builtin_amdgcn_sched_barrier(0);
     }
 }
 
-// relu(acc) of NB row blocks -> B fragments of the next layer
-template <int PREC, int NB>
-__device__ __forceinline__ void relu_to_frags(const floatx16 *acc, typename Mma<PREC>::frag (*out)[Mma<PREC>::NP]) {
-    // out points at the first fragment of the first of the NB row blocks
-    using M = Mma<PREC>;
-    constexpr int G = M::G;
-#pragma unroll
-    for (int fb = 0; fb < NB; ++fb) {
-        float hv[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) hv[v] = fmaxf(acc[fb][v], 0.0f);
-#pragma unroll
-        for (int u = 0; u < 16 / G; ++u) M::pack(hv + u * G, out[fb * (16 / G) + u]);
-    }
+// max(x, 0) for finite floats as one integer instruction (negative floats are negative integers)
+__device__ __forceinline__ float relu_f32(float x) {
+    return __builtin_bit_cast(float, max(__builtin_bit_cast(int, x), 0));
 }
 
-// raw[16] (lane's 16 row values, view direction already inserted) -> rgb of the lane's
-// sample in out[0..2] (meaningful on lanes with h == 0)
+// relu(acc) of one row block -> G-slot B fragments of the next layer
 template <int PREC>
+__device__ __forceinline__ void relu_to_frags(const floatx16 &acc, typename Mma<PREC>::frag (*out)[Mma<PREC>::NP]) {
+    using M = Mma<PREC>;
+    constexpr int G = M::G;
+    float hv[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) hv[v] = relu_f32(acc[v]);
+#pragma unroll
+    for (int u = 0; u < 16 / G; ++u) M::pack(hv + u * G, out[u]);
+}
+
+// raw[cb][16] (the lane's 16 input rows of each of its NCB samples) -> rgb in out[cb][0..2]
+// (meaningful on lanes with h == 0)
+template <int PREC, int NCB>
 __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w1, const typename Mma<PREC>::frag *w2,
                                                const typename Mma<PREC>::frag *w3, const float *b1, const float *b2,
-                                               const float *b3, const float *raw, unsigned lane, float *out) {
+                                               const float *b3, const float (*raw)[16], unsigned lane, float (*out)[3]) {
     using M = Mma<PREC>;
     using frag = typename M::frag;
     constexpr int G = M::G, NP = M::NP;
     constexpr int T1 = kSlots1 / G, T2 = 64 / G;
+    constexpr int NB = NCB == 1 ? 4 : 2;  // row blocks per pass: NB*NCB accumulators of 16 registers
+    constexpr int PF = G == 1 ? 4 : 1;
     const unsigned h = lane >> 5;
-    frag b2frag[T2][NP];
+    frag b2frag[NCB][T2][NP];
     {
-        frag bfrag[T1][NP];
-        {
+        frag bfrag[NCB][T1][NP];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
             float slots[kSlots1];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float x = raw[v];
+                const float x = raw[cb][v];
                 float s1, c1;
                 if (PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2) {
                     sincos_f32(x, s1, c1);
@@ -247,33 +262,44 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
                 slots[v] = x; slots[16 + v] = s1; slots[32 + v] = c1; slots[48 + v] = s2; slots[64 + v] = c2;
             }
 #pragma unroll
-            for (int t = 0; t < T1; ++t) M::pack(slots + t * G, bfrag[t]);
+            for (int t = 0; t < T1; ++t) M::pack(slots + t * G, bfrag[cb][t]);
         }
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {  // two row blocks at a time: 32 accumulator registers
-            floatx16 acc[2];
-            acc[0] = load_bias(b1, (2 * half) * 2 + h);
-            acc[1] = load_bias(b1, (2 * half + 1) * 2 + h);
-            dense_layer<PREC, 2, T1>(w1, 2 * half, lane, bfrag, acc);
-            relu_to_frags<PREC, 2>(acc, b2frag + 2 * half * (16 / G));
-        }
-    }
-    frag b3frag[T2][NP];
-    {
+        for (int pass = 0; pass < 4 / NB; ++pass) {
+            floatx16 acc[NB][NCB];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            floatx16 acc[2];
-            acc[0] = load_bias(b2, (2 * half) * 2 + h);
-            acc[1] = load_bias(b2, (2 * half + 1) * 2 + h);
-            dense_layer<PREC, 2, T2>(w2, 2 * half, lane, b2frag, acc);
-            relu_to_frags<PREC, 2>(acc, b3frag + 2 * half * (16 / G));
+            for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) acc[fb][cb] = load_bias(b1, (pass * NB + fb) * 2 + h);
+            dense_layer<PREC, NB, NCB, T1, PF>(w1, pass * NB, lane, bfrag, acc);
+#pragma unroll
+            for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+                for (int cb = 0; cb < NCB; ++cb) relu_to_frags<PREC>(acc[fb][cb], &b2frag[cb][(pass * NB + fb) * (16 / G)]);
         }
     }
-    floatx16 acc3[1];
-    acc3[0] = load_bias(b3, h);
-    dense_layer<PREC, 1, T2>(w3, 0, lane, b3frag, acc3);
+    frag b3frag[NCB][T2][NP];
 #pragma unroll
-    for (int k = 0; k < 3; ++k) out[k] = 1.0f / (1.0f + expf(-acc3[0][k]));
+    for (int pass = 0; pass < 4 / NB; ++pass) {
+        floatx16 acc[NB][NCB];
+#pragma unroll
+        for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) acc[fb][cb] = load_bias(b2, (pass * NB + fb) * 2 + h);
+        dense_layer<PREC, NB, NCB, T2, PF>(w2, pass * NB, lane, b2frag, acc);
+#pragma unroll
+        for (int fb = 0; fb < NB; ++fb)
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) relu_to_frags<PREC>(acc[fb][cb], &b3frag[cb][(pass * NB + fb) * (16 / G)]);
+    }
+    floatx16 acc3[1][NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) acc3[0][cb] = load_bias(b3, h);
+    dense_layer<PREC, 1, NCB, T2, (G == 1 ? 8 : 4)>(w3, 0, lane, b3frag, acc3);
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) out[cb][k] = 1.0f / (1.0f + expf(-acc3[0][cb][k]));
 }
 
 template <int PREC> struct LdsPlan {
@@ -282,7 +308,9 @@ template <int PREC> struct LdsPlan {
     static constexpr size_t kW2 = (size_t)4 * 64 * 64 * sizeof(typename M::elem) * M::NP;
     static constexpr size_t kW3 = (size_t)64 * 64 * sizeof(typename M::elem) * M::NP;
     static constexpr bool kW3InLds = (kW1 + kW2 + kW3) <= 96 * 1024;
-    static constexpr size_t kBytes = kW1 + kW2 + (kW3InLds ? kW3 : 0);
+    static constexpr size_t kBias = (4 * 2 * 16 + 4 * 2 * 16 + 2 * 16) * sizeof(float);  // b1 | b2 | b3, register order
+    static constexpr size_t kWeights = kW1 + kW2 + (kW3InLds ? kW3 : 0);
+    static constexpr size_t kBytes = kWeights + kBias;
 };
 
 template <int PREC>
@@ -298,6 +326,11 @@ __device__ __forceinline__ void stage_weights(char *lds, const char *packed, con
     d += P::kW2 / 16;
     if (P::kW3InLds)
         for (size_t i = threadIdx.x; i < P::kW3 / 16; i += blockDim.x) d[i] = s3[i];
+    // biases: read once per layer and row block by every wave, so they live next to the weights
+    float *bl = reinterpret_cast<float *>(lds + P::kWeights);
+    const float *b1 = (const float *)(packed + L.b1), *b2 = (const float *)(packed + L.b2), *b3 = (const float *)(packed + L.b3);
+    for (unsigned i = threadIdx.x; i < 128; i += blockDim.x) { bl[i] = b1[i]; bl[128 + i] = b2[i]; }
+    for (unsigned i = threadIdx.x; i < 32; i += blockDim.x) bl[256 + i] = b3[i];
     __syncthreads();
 }
 
@@ -318,32 +351,51 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
     const frag *w2 = reinterpret_cast<const frag *>(lds + P::kW1);
     const frag *w3 = P::kW3InLds ? reinterpret_cast<const frag *>(lds + P::kW1 + P::kW2)
                                  : reinterpret_cast<const frag *>(packed + L.w3);
-    const float *b1 = (const float *)(packed + L.b1), *b2 = (const float *)(packed + L.b2),
-                *b3 = (const float *)(packed + L.b3);
+    const float *b1 = reinterpret_cast<const float *>(lds + P::kWeights), *b2 = b1 + 128, *b3 = b1 + 256;
     const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
     const uint64_t M = MODE == 0 ? M_host : (uint64_t)*count;
-    const uint64_t n_tiles = (M + 31) / 32;
+    constexpr int NCB = MlpBlock<PREC>::NCB, TILE = 32 * NCB;
+    const uint64_t n_tiles = (M + TILE - 1) / TILE;
     const unsigned wpb = MlpBlock<PREC>::N / LM_WAVE;
     const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * wpb + threadIdx.x / LM_WAVE;
     const uint64_t n_waves = (uint64_t)gridDim.x * wpb;
-    for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
-        const uint64_t p = tile * 32 + j;
-        const bool live = p < M;
-        const uint64_t pc = live ? p : M - 1;
-        const float *vsrc = MODE == 0 ? view + pc * 3 : view + 6 * (size_t)(app_idx[pc] / (uint32_t)S) + 3;
-        float raw[16];
+    // the lane's 16 input rows (features, view direction, zeros) of its sample in each column block
+    auto fetch = [&](uint64_t tile, float (*raw)[16]) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = row_of(v, (int)h);
-            float x = 0.0f;
-            if (row < kAppDim) x = feat[pc * kAppDim + row];
-            else if (row >= 28 && row <= 30) x = vsrc[row - 28];
-            raw[v] = x;
+        for (int cb = 0; cb < NCB; ++cb) {
+            const uint64_t p = tile * TILE + cb * 32 + j;
+            const uint64_t pc = p < M ? p : M - 1;
+            const float *f = feat + pc * kAppDim;
+            const float *vsrc = MODE == 0 ? view + pc * 3 : view + 6 * (size_t)(app_idx[pc] / (uint32_t)S) + 3;
+#pragma unroll
+            for (int v = 0; v < 15; ++v) {
+                // both halves' rows are compile-time constants: pick the address, load unconditionally
+                const int r0 = row_of(v, 0), r1 = row_of(v, 1);
+                const float *a0 = f + r0;
+                const float *a1 = r1 < kAppDim ? f + r1 : vsrc + (r1 - 28);
+                raw[cb][v] = *(h ? a1 : a0);
+            }
+            raw[cb][15] = 0.0f;
         }
-        float out[3];
-        colour_network<PREC>(w1, w2, w3, b1, b2, b3, raw, lane, out);
-        if (live && h == 0) {
-            rgb[p * 3 + 0] = out[0]; rgb[p * 3 + 1] = out[1]; rgb[p * 3 + 2] = out[2];
+    };
+    float nxt[NCB][16];
+    if (wave_id < n_tiles) fetch(wave_id, nxt);
+    for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
+        float raw[NCB][16];
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) raw[cb][v] = nxt[cb][v];
+        // the next tile's inputs travel while this tile is multiplied
+        if (tile + n_waves < n_tiles) fetch(tile + n_waves, nxt);
+        float out[NCB][3];
+        colour_network<PREC, NCB>(w1, w2, w3, b1, b2, b3, raw, lane, out);
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) {
+            const uint64_t p = tile * TILE + cb * 32 + j;
+            if (p < M && h == 0) {
+                rgb[p * 3 + 0] = out[cb][0]; rgb[p * 3 + 1] = out[cb][1]; rgb[p * 3 + 2] = out[cb][2];
+            }
         }
     }
 }
@@ -477,7 +529,7 @@ extern "C" int lm_mlp_pack_bias1(const float *b1, float *packed_b1_out) {
 }
 
 static unsigned mlp_grid(uint64_t M) {
-    const uint64_t tiles = (M + 31) / 32, wpb = 4, blocks = (tiles + wpb - 1) / wpb;
+    const uint64_t tiles = (M + 63) / 64, wpb = 4, blocks = (tiles + wpb - 1) / wpb;
     return (unsigned)std::min<uint64_t>(std::max<uint64_t>(blocks, 1), (uint64_t)lm_persistent_blocks(1));
 }
 
