@@ -37,7 +37,6 @@ MLP_FLOP_PER_ROW = 2 * (150 * 128 + 128 * 128 + 128 * 3)
 # kernels at the default chunk size; any other configuration reports null.
 MEASURED_TRAFFIC = {
     ("c4_1080p_multires_P3_base1024_shift0", 262144, "k_app_feat"): 4.17e9 + 0.10e9,
-    ("c4_1080p_multires_P3_base1024_shift0", 262144, "k_density_list"): 4.93e9 + 0.01e9,
 }
 
 
@@ -74,7 +73,9 @@ def bench_frame(args, workload):
         name = f"c5_4k_cityblock_res{args.base * 8}"
     else:
         raise ValueError(workload)
-    model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=args.term_eps)
+    term_eps = 1e-4 / float(p.near_far[1]) if args.term_eps == "auto" else float(args.term_eps)
+    args.term_eps = term_eps
+    model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=term_eps)
     torch.cuda.synchronize()
     log(f"[bench] scene {name} built in {time.time() - t0:.1f}s; tables "
         f"{sum(t.numel() * t.element_size() for t in model._tables) / 1e9:.2f} GB")
@@ -113,6 +114,7 @@ def bench_frame(args, workload):
 
     cnt = counters.cpu().long() & 0xFFFFFFFF
     n_valid, n_app = int(cnt[:, L.LM_STAT_N_VALID].sum()), int(cnt[:, L.LM_STAT_N_APP].sum())
+    n_marched = int(cnt[:, L.LM_STAT_N_MARCHED].sum())
     stage_ms = [0.0] * L.LM_N_STAGES  # per frame, averaged over steps
     for per_step in events:
         for per_chunk in per_step:
@@ -120,20 +122,21 @@ def bench_frame(args, workload):
                 stage_ms[s] += per_chunk[s].elapsed_time(per_chunk[s + 1])
     stage_ms = [x / args.steps for x in stage_ms]
     launches = n_chunks  # one launch of each stage kernel per chunk
-    dens_B = plane_bytes_per_sample(model._density) + 8  # + list index in, sigma out
+    dens_B = plane_bytes_per_sample(model._density) + 4  # + weight out
     app_B = plane_bytes_per_sample(model._app) + 4 + 27 * 4  # + index in, projected features out
     stages = {}
     for i, nm in enumerate(L.STAGE_NAMES):
         stages[nm] = {"ms_per_frame": round(stage_ms[i], 4)}
-    stages["density"].update(bytes_per_sample=dens_B, GBps=round(n_valid * dens_B / (stage_ms[1] * 1e-3) / 1e9, 1))
+    stages["density_march"].update(bytes_per_sample=dens_B, samples=n_marched,
+                                   GBps=round(n_marched * dens_B / (stage_ms[1] * 1e-3) / 1e9, 1))
     stages["app_gather"].update(bytes_per_sample=app_B, GBps=round(n_app * app_B / max(stage_ms[3], 1e-9) / 1e6, 1))
     stages["colour"].update(TFLOPs=round(n_app * (MLP_FLOP_PER_ROW + 2 * model.K_app * 27) / max(stage_ms[4], 1e-9) / 1e9, 2))
     cull_B = 32 + 0.125  # 8 corner loads of the float volume per in-box sample (upper bound: every sample), bitmap out
     stages["cull"].update(GBps=round((N * S * cull_B + n_valid * 4) / (stage_ms[0] * 1e-3) / 1e9, 1))
-    stages["weights"].update(GBps=round((n_valid * 4 + N * S / 8 + n_app * 8 + N * 8) / (stage_ms[2] * 1e-3) / 1e9, 1))
+    stages["app_list"].update(GBps=round((n_marched * 4 + N * S / 8 + n_app * 8 + N * 16) / (stage_ms[2] * 1e-3) / 1e9, 1))
 
     # dominant kernel -> roofline object
-    cand = {"density": stage_ms[1], "app_gather": stage_ms[3], "colour": stage_ms[4]}
+    cand = {"density_march": stage_ms[1], "app_gather": stage_ms[3], "colour": stage_ms[4]}
     dom = max(cand, key=cand.get)
     if dom == "colour":
         ach = stages["colour"]["TFLOPs"]
@@ -142,7 +145,7 @@ def bench_frame(args, workload):
                 "frac": round(ach / peak, 4), "traffic": None}
     else:
         ach = stages[dom]["GBps"]
-        roof = {"kernel": "k_density_list" if dom == "density" else "k_app_feat", "bound": "hbm", "achieved": ach,
+        roof = {"kernel": "k_march" if dom == "density_march" else "k_app_feat", "bound": "hbm", "achieved": ach,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
     roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
     roof["launches_per_frame"] = launches
@@ -156,9 +159,10 @@ def bench_frame(args, workload):
         "scaling": "weak", "vs_baseline": None, "dtype": "f32" if args.mlp == "f32" else f"f32+{args.mlp}-mlp",
         "data": "synthetic",
         "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "mlp": args.mlp,
-                   "term_eps": args.term_eps, "valid_samples": n_valid, "app_samples": n_app},
+                   "term_eps": args.term_eps, "valid_samples": n_valid, "marched_samples": n_marched, "app_samples": n_app},
         "frames_per_s": round(1e3 / ms_step, 3), "mpixel_per_s": round(mrays, 3),
-        "gather_GBps": stages["density"]["GBps"], "gather_frac_of_hbm_peak": round(stages["density"]["GBps"] / HBM_PEAK_GBS, 4),
+        "gather_GBps": stages["density_march"]["GBps"],
+        "gather_frac_of_hbm_peak": round(stages["density_march"]["GBps"] / HBM_PEAK_GBS, 4),
         "stages": stages, "roofline": roof, "cpu_baseline": cpu, "parity": parity,
     }
     return out
@@ -306,7 +310,9 @@ def main():
     ap.add_argument("--frame", type=int, default=0)
     ap.add_argument("--density-shift", type=float, default=0.0)
     ap.add_argument("--mlp", default="f16x2", choices=["f32", "f16x2", "f16", "bf16"])
-    ap.add_argument("--term-eps", type=float, default=0.0)
+    ap.add_argument("--term-eps", default="auto",
+                    help="ray termination threshold on the transmittance; 'auto' = 1e-4 / far, the largest value that "
+                         "keeps rgb and depth within 1e-4 of the unterminated render; 0 = never terminate")
     ap.add_argument("--chunk", type=int, default=262144)
     ap.add_argument("--queries", type=int, default=1 << 24)
     ap.add_argument("--rows", type=int, default=1 << 23)

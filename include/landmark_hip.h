@@ -94,9 +94,9 @@ typedef struct lm_geom {
 
 /* stages of lm_render, in launch order */
 enum {
-    LM_STAGE_CULL = 1,      /* sampling + culling + compaction (3 kernels) */
-    LM_STAGE_DENSITY = 2,   /* density gather over the valid list */
-    LM_STAGE_WEIGHTS = 3,   /* per-ray scan, appearance list */
+    LM_STAGE_CULL = 1,      /* sampling + culling + compaction, list of rays with valid samples */
+    LM_STAGE_DENSITY = 2,   /* density gather fused with the per-ray transmittance march */
+    LM_STAGE_WEIGHTS = 3,   /* appearance list from the stored weights */
     LM_STAGE_APP = 4,       /* appearance gather */
     LM_STAGE_COLOUR = 5,    /* basis_mat + encoding + colour network */
     LM_STAGE_COMPOSITE = 6, /* per-ray colour sum */
@@ -127,7 +127,9 @@ typedef struct lm_model {
 } lm_model;
 
 /* Counters written by lm_render (device memory, 8 x uint32). */
-enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_WORDS = 8 };
+/* N_ACTIVE: rays with at least one valid sample; QUEUE: internal work-queue cursor;
+ * N_MARCHED: valid samples whose density was gathered (< N_VALID with early termination) */
+enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_ACTIVE = 2, LM_STAT_QUEUE = 3, LM_STAT_N_MARCHED = 4, LM_STAT_WORDS = 8 };
 
 int lm_abi_version(void);
 const char *lm_last_error(void);

@@ -80,6 +80,15 @@ int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float
 int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
                         const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream);
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
+int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *ray_list,
+                          uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt, uint32_t *p_end,
+                          hipStream_t stream);
+int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, const float *w_valid,
+                        float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
+                        uint32_t *app_idx, float *app_w, uint32_t *app_count, hipStream_t stream);
+int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *word_prefix,
+                    const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
+                    float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st);
 int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
                     float *feat, hipStream_t st);
 
@@ -93,6 +102,8 @@ struct Workspace {
     float *w_valid;
     uint32_t *app_first;
     uint32_t *app_cnt;
+    uint32_t *p_end;
+    uint32_t *ray_list;
     uint32_t *app_idx;
     float *app_w;
     float *rgb;
@@ -122,6 +133,8 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products)
     w.w_valid = (float *)take(total * 4);
     w.app_first = (uint32_t *)take((uint64_t)N * 4);
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
+    w.p_end = (uint32_t *)take((uint64_t)N * 4);
+    w.ray_list = (uint32_t *)take((uint64_t)N * 4);
     w.app_idx = (uint32_t *)take(cap * 4);
     w.app_w = (float *)take(cap * 4);
     w.rgb = (float *)take(cap * 12);
@@ -173,12 +186,16 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
     if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, w.valid_idx, cnt, nullptr, w.cull_scratch, st))
         return rc;
+    if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.ray_list, cnt + LM_STAT_N_ACTIVE, w.acc, depth_map,
+                                       w.app_cnt, w.p_end, st))
+        return rc;
     mark(LM_STAGE_CULL);
-    if (int rc = lm_density_valid(m, rays, w.valid_idx, cnt, w.sigma, st)) return rc;
+    if (int rc = lm_launch_march(m, rays, w.bitmap, w.word_prefix, w.ray_list, cnt + LM_STAT_N_ACTIVE, cnt + LM_STAT_QUEUE,
+                                 w.w_valid, w.acc, depth_map, w.app_cnt, w.p_end, cnt + LM_STAT_N_MARCHED, st))
+        return rc;
     mark(LM_STAGE_DENSITY);
-    if (int rc = lm_weights(&m->geom, rays, N, w.bitmap, w.word_prefix, w.sigma, m->distance_scale, m->weight_thres,
-                            m->term_eps, w.w_valid, nullptr, w.app_first, w.app_cnt, w.app_idx, w.app_w, w.acc, depth_map,
-                            cnt, st))
+    if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.word_prefix, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
+                                     w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, st))
         return rc;
     mark(LM_STAGE_WEIGHTS);
     if (fused) {

@@ -166,3 +166,40 @@ __device__ __forceinline__ unsigned lm_lane() { return __lane_id(); }
 __device__ __forceinline__ unsigned lm_mbcnt(uint64_t mask) {  // set bits of mask below this lane
     return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
+
+// Iterates the set bits of the sample bitmap in [flat0, flat1): the valid samples of one ray.
+struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
+    const uint64_t *bitmap;
+    const uint32_t *prefix;
+    uint64_t w, w_last, bits, flat1;
+    uint32_t pos;
+    __device__ __forceinline__ void start(const uint64_t *bm, const uint32_t *pf, uint64_t flat0, uint64_t flat1_) {
+        bitmap = bm; prefix = pf; flat1 = flat1_;
+        w = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
+        const uint64_t raw = bm[w];
+        const unsigned b0 = (unsigned)(flat0 & 63);
+        const uint64_t below = b0 ? ((1ull << b0) - 1ull) : 0ull;
+        pos = pf[w] + (uint32_t)__popcll(raw & below);
+        bits = mask_tail(raw & ~below);
+    }
+    __device__ __forceinline__ uint64_t mask_tail(uint64_t x) const {
+        if (w == w_last) {
+            const unsigned e = (unsigned)(flat1 & 63);
+            if (e) x &= (1ull << e) - 1ull;
+        }
+        return x;
+    }
+    // next set bit -> flat index; false when exhausted.  `pos` is the compact position of it.
+    __device__ __forceinline__ bool next(uint64_t &flat) {
+        while (bits == 0) {
+            if (w == w_last) return false;
+            ++w;
+            bits = mask_tail(bitmap[w]);
+        }
+        const int b = __ffsll((unsigned long long)bits) - 1;
+        bits &= bits - 1;
+        flat = w * 64 + (uint64_t)b;
+        return true;
+    }
+};
+

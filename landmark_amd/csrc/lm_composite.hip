@@ -21,41 +21,6 @@ namespace {
 
 constexpr int kBlock = 256;
 
-struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
-    const uint64_t *bitmap;
-    const uint32_t *prefix;
-    uint64_t w, w_last, bits, flat1;
-    uint32_t pos;
-    __device__ __forceinline__ void start(const uint64_t *bm, const uint32_t *pf, uint64_t flat0, uint64_t flat1_) {
-        bitmap = bm; prefix = pf; flat1 = flat1_;
-        w = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
-        const uint64_t raw = bm[w];
-        const unsigned b0 = (unsigned)(flat0 & 63);
-        const uint64_t below = b0 ? ((1ull << b0) - 1ull) : 0ull;
-        pos = pf[w] + (uint32_t)__popcll(raw & below);
-        bits = mask_tail(raw & ~below);
-    }
-    __device__ __forceinline__ uint64_t mask_tail(uint64_t x) const {
-        if (w == w_last) {
-            const unsigned e = (unsigned)(flat1 & 63);
-            if (e) x &= (1ull << e) - 1ull;
-        }
-        return x;
-    }
-    // next set bit -> flat index; false when exhausted.  `pos` is the compact position of it.
-    __device__ __forceinline__ bool next(uint64_t &flat) {
-        while (bits == 0) {
-            if (w == w_last) return false;
-            ++w;
-            bits = mask_tail(bitmap[w]);
-        }
-        const int b = __ffsll((unsigned long long)bits) - 1;
-        bits &= bits - 1;
-        flat = w * 64 + (uint64_t)b;
-        return true;
-    }
-};
-
 __global__ __launch_bounds__(kBlock) void k_weights(lm_geom g, const float *__restrict__ rays, uint64_t N,
                                                     const uint64_t *__restrict__ bitmap,
                                                     const uint32_t *__restrict__ word_prefix,
@@ -160,6 +125,76 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
     rgb_map[3 * r + 2] = fminf(fmaxf(c2, 0.0f), 1.0f);
 }
 
+// Rays that have at least one valid sample, for the marching kernel's queue; the others get
+// their (zero) results here.
+__global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
+                                                        const uint32_t *__restrict__ word_prefix,
+                                                        uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
+                                                        float *__restrict__ acc, float *__restrict__ depth,
+                                                        uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end) {
+    const unsigned lane = lm_lane();
+    const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    bool any = false;
+    if (r < N) {
+        BitWalk it;
+        it.start(bitmap, word_prefix, r * (uint64_t)S, (r + 1) * (uint64_t)S);
+        uint64_t flat;
+        any = it.next(flat);
+        if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = it.pos; }
+    }
+    const uint64_t mask = __ballot(any);
+    if (mask) {
+        uint32_t base = 0;
+        if (lane == 0) base = atomicAdd(n_active, (uint32_t)__popcll(mask));
+        base = __shfl(base, 0);
+        if (any) ray_list[base + lm_mbcnt(mask)] = (uint32_t)r;
+    }
+}
+
+// Appearance list from stored weights: a contiguous slot range per ray (wave prefix + one
+// atomic), filled in sample order from the weights of the ray's samples [first, p_end).
+__global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
+                                                      const uint32_t *__restrict__ word_prefix,
+                                                      const float *__restrict__ w_valid, float weight_thres,
+                                                      const uint32_t *__restrict__ app_cnt,
+                                                      const uint32_t *__restrict__ p_end,
+                                                      uint32_t *__restrict__ app_first, uint32_t *__restrict__ app_idx,
+                                                      float *__restrict__ app_w, uint32_t *__restrict__ app_count) {
+    const unsigned lane = lm_lane();
+    const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t cnt = r < N ? app_cnt[r] : 0;
+    uint32_t incl = cnt;
+#pragma unroll
+    for (int d = 1; d < LM_WAVE; d <<= 1) {
+        const uint32_t y = __shfl_up(incl, d);
+        if (lane >= (unsigned)d) incl += y;
+    }
+    const uint32_t total = __shfl(incl, LM_WAVE - 1);
+    uint32_t base = 0;
+    if (total) {
+        if (lane == 0) base = atomicAdd(app_count, total);
+        base = __shfl(base, 0);
+    }
+    if (r >= N) return;
+    uint32_t slot = base + incl - cnt;
+    app_first[r] = slot;
+    if (cnt) {
+        BitWalk it;
+        it.start(bitmap, word_prefix, r * (uint64_t)S, (r + 1) * (uint64_t)S);
+        const uint32_t end = p_end[r];
+        uint64_t flat;
+        for (uint32_t p = it.pos; p < end; ++p) {
+            it.next(flat);
+            const float wgt = w_valid[p];
+            if (wgt > weight_thres) {
+                app_idx[slot] = (uint32_t)flat;
+                app_w[slot] = wgt;
+                ++slot;
+            }
+        }
+    }
+}
+
 __global__ void k_zero_counters(uint32_t *c) {
     if (threadIdx.x < LM_STAT_WORDS) c[threadIdx.x] = 0;
 }
@@ -199,5 +234,25 @@ int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *ap
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
     hipLaunchKernelGGL(k_zero_counters, dim3(1), dim3(64), 0, stream, counters);
     LM_CHECK_LAUNCH("k_zero_counters");
+    return LM_OK;
+}
+
+int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *ray_list,
+                          uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt, uint32_t *p_end,
+                          hipStream_t stream) {
+    const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(k_active_rays, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, ray_list,
+                       n_active, acc, depth, app_cnt, p_end);
+    LM_CHECK_LAUNCH("k_active_rays");
+    return LM_OK;
+}
+
+int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, const float *w_valid,
+                        float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
+                        uint32_t *app_idx, float *app_w, uint32_t *app_count, hipStream_t stream) {
+    const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
+    hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, w_valid,
+                       weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count);
+    LM_CHECK_LAUNCH("k_app_slots");
     return LM_OK;
 }

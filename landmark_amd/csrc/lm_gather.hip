@@ -258,6 +258,103 @@ __global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int
 }
 
 
+// ---- density gather fused with the transmittance march ------------------------------------
+// Four lanes (a quad) own one ray at a time and walk its valid samples in order: gather the
+// density of the next sample (each lane a quarter of the channels), turn it into alpha and a
+// weight, carry the transmittance along.  Quads take rays from a queue of the rays that have
+// valid samples and fetch a new one as soon as theirs ends, so the sixteen quads of a wave
+// stay busy whatever the rays' lengths.  Two things follow from walking rays in lock step:
+// neighbouring rays are at similar depths in the same load instruction, so their corner
+// texels share cache lines; and a ray can stop once its transmittance is below term_eps,
+// before the density of the samples behind is ever fetched.  With term_eps = 0 the weights
+// are those of the separate density + weights kernels, bit for bit (same operations, and the
+// transmittance is the same sequential product torch.cumprod forms, app/tools/utils.py:51-64).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
+                                                  const float *__restrict__ rays, const uint64_t *__restrict__ bitmap,
+                                                  const uint32_t *__restrict__ word_prefix,
+                                                  const uint32_t *__restrict__ ray_list,
+                                                  const uint32_t *__restrict__ n_active_ptr, uint32_t *__restrict__ queue,
+                                                  int act, float shift, float distance_scale, float weight_thres,
+                                                  float term_eps, float *__restrict__ w_valid,
+                                                  float *__restrict__ acc_out, float *__restrict__ depth_out,
+                                                  uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end_out,
+                                                  uint32_t *__restrict__ n_marched) {
+    const unsigned lane = lm_lane(), qlane = lane & 3u, leader = lane & ~3u;
+    uint32_t marched = 0;  // samples whose density this lane's quad gathered (statistics)
+    const uint32_t n_active = *n_active_ptr;
+    const int S = g.S;
+    bool have = false, done = false;
+    uint32_t r = 0, p = 0, cnt = 0;
+    uint64_t flat0 = 0;
+    float ray[6] = {0, 0, 0, 0, 0, 0}, rp = 0.0f, Tr = 1.0f, acc = 0.0f, depth = 0.0f;
+    BitWalk it;
+    it.bits = 0; it.w = it.w_last = 0; it.flat1 = 0; it.pos = 0; it.bitmap = bitmap; it.prefix = word_prefix;
+    while (true) {
+        // quads without a ray take the next ones from the queue: one atomic per wave and round
+        const bool need = !have && !done;
+        const uint64_t need_mask = __ballot(need && qlane == 0);
+        if (need_mask) {
+            const int first = __ffsll((unsigned long long)need_mask) - 1;
+            uint32_t base = 0;
+            if ((int)lane == first) base = atomicAdd(queue, (uint32_t)__popcll(need_mask));
+            base = __shfl(base, first);
+            if (need) {
+                const uint32_t idx = base + (uint32_t)__popcll(need_mask & ((1ull << leader) - 1ull));
+                if (idx >= n_active) {
+                    done = true;
+                } else {
+                    r = ray_list[idx];
+                    const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
+                    const float2 a = rp2[0], b = rp2[1], c = rp2[2];
+                    ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+                    rp = lm_ray_param(g, ray);
+                    flat0 = (uint64_t)r * (uint64_t)S;
+                    it.start(bitmap, word_prefix, flat0, flat0 + S);
+                    p = it.pos;
+                    Tr = 1.0f; acc = 0.0f; depth = 0.0f; cnt = 0;
+                    have = true;
+                }
+            }
+        }
+        if (!__any(have)) break;
+        if (have) {
+            uint64_t flat;
+            bool finish = !it.next(flat);
+            if (!finish) {
+                const int s = (int)(flat - flat0);
+                const float z = lm_sample_z(g, rp, s);
+                float pt[3], q[3];
+                lm_point(ray, z, pt);
+                lm_normalise(g, pt, q);
+                const float sig = activate(density_sum<T>(ps, q, qlane, den_w), act, shift);
+                const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
+                const float d2 = dist * distance_scale;
+                const float alpha = 1.0f - expf(-sig * d2);
+                const float wgt = alpha * Tr;
+                Tr = Tr * ((1.0f - alpha) + 1e-10f);
+                if (qlane == 0) w_valid[p] = wgt;
+                acc += wgt;
+                depth += wgt * z;
+                cnt += wgt > weight_thres;
+                ++p;
+                ++marched;
+                finish = term_eps > 0.0f && Tr < term_eps;
+            }
+            if (finish) {
+                if (qlane == 0) {
+                    acc_out[r] = acc; depth_out[r] = depth; app_cnt[r] = cnt; p_end_out[r] = p;
+                }
+                have = false;
+            }
+        }
+    }
+    if (qlane != 0) marched = 0;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) marched += __shfl_xor(marched, d);
+    if (lane == 0 && marched) atomicAdd(n_marched, marched);
+}
+
 // ---- appearance gather fused with basis_mat --------------------------------------------------
 // One wave owns 32 appearance samples; lane (j, h) gathers, for sample j, CW consecutive
 // channels of every group of 2*CW (the lane pair of a sample covers the group), multiplies
@@ -565,4 +662,25 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
         default: LM_AF_GO(LM_MLP_F16X2);
     }
 #undef LM_AF_GO
+}
+
+// Density + transmittance march over the rays listed in ray_list (those with valid samples).
+int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *word_prefix,
+                    const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
+                    float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st) {
+    int dtype;
+    if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
+    LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
+    const PlaneSet ps = make_set(m->density, m->n_planes);
+    const unsigned grid = (unsigned)lm_persistent_blocks(8);
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_march<float>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
+                           word_prefix, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
+                           m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
+    else
+        hipLaunchKernelGGL(k_march<__half>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
+                           word_prefix, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
+                           m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
+    LM_CHECK_LAUNCH("k_march");
+    return LM_OK;
 }
