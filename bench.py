@@ -317,7 +317,7 @@ def main():
     ap.add_argument("--queries", type=int, default=1 << 24)
     ap.add_argument("--rows", type=int, default=1 << 23)
     ap.add_argument("--coherent", action="store_true")
-    ap.add_argument("--cpu-rows", type=int, default=8)
+    ap.add_argument("--cpu-rows", type=int, default=270)
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calib", action="store_true", help="also run one 1 GiB device copy (counter calibration)")

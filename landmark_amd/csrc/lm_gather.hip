@@ -151,6 +151,39 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
     return den_w ? fmaxf(sum, 0.0f) : sum;
 }
 
+// Same sum with a compile-time channel count shared by all planes: the channel groups of a
+// plane are unrolled, so a lane has 6 * C / (4 V) independent loads in flight per plane
+// instead of 6 (wide planes, e.g. the 64-channel isolated-gather configuration).
+template <typename T, int C>
+__device__ __forceinline__ float density_sum_fixed(const PlaneSet &ps, const float *q, unsigned qlane,
+                                                   const float *__restrict__ den_w) {
+    constexpr int V = Vec<T>::V;
+    constexpr int NG = (C + V * kQuad - 1) / (V * kQuad);
+    float sum = 0.0f;
+    for (int k = 0; k < ps.n; ++k) {
+        const lm_plane &pl = ps.p[k];
+        const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+        const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        float prod[NG][V];
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+            const int c = V * (int)qlane + gi * V * kQuad;
+            plane_products<T>(pl, t2, t1, c < C ? c : C - V, prod[gi]);
+        }
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+            const int c = V * (int)qlane + gi * V * kQuad;
+            if (c < C) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) sum = den_w ? fmaf(den_w[k * C + c + i], prod[gi][i], sum) : sum + prod[gi][i];
+            }
+        }
+    }
+    sum += __shfl_xor(sum, 1);
+    sum += __shfl_xor(sum, 2);
+    return den_w ? fmaxf(sum, 0.0f) : sum;
+}
+
 template <typename T>
 __device__ __forceinline__ void app_store(const PlaneSet &ps, const float *q, unsigned qlane, float *row) {
     constexpr int V = Vec<T>::V;
@@ -193,7 +226,7 @@ __device__ __forceinline__ float activate(float f, int act, float shift) {
 }
 
 // ---- explicit coordinates ----------------------------------------------------------------
-template <typename T>
+template <typename T, int CFIX>  // CFIX > 0: every plane has CFIX channels
 __global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float *__restrict__ den_w,
                                                         const float *__restrict__ xyz, uint64_t M,
                                                         float *__restrict__ out) {
@@ -203,7 +236,8 @@ __global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float
         const uint64_t p = tile * kTile + slot;
         if (p >= M) continue;
         float q[3] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2]};
-        const float s = density_sum<T>(ps, q, qlane, den_w);
+        const float s = CFIX > 0 ? density_sum_fixed<T, (CFIX > 0 ? CFIX : 16)>(ps, q, qlane, den_w)
+                                 : density_sum<T>(ps, q, qlane, den_w);
         if (qlane == 0) out[p] = s;
     }
 }
@@ -555,12 +589,17 @@ extern "C" int lm_gather_density_xyz(const lm_plane *planes, int32_t n_planes, c
     const PlaneSet ps = make_set(planes, n_planes);
     const uint64_t tiles = ((uint64_t)M + kTile - 1) / kTile;
     const unsigned grid = (unsigned)std::min<uint64_t>(tiles, (uint64_t)lm_persistent_blocks(8));
-    if (dtype == LM_F32)
-        hipLaunchKernelGGL(k_density_xyz<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, density_basis, xyz,
-                           (uint64_t)M, out);
-    else
-        hipLaunchKernelGGL(k_density_xyz<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, density_basis, xyz,
-                           (uint64_t)M, out);
+    bool all64 = true;
+    for (int k = 0; k < n_planes; ++k) all64 &= planes[k].C == 64;
+#define LM_DX(T_, C_)                                                                                               \
+    hipLaunchKernelGGL((k_density_xyz<T_, C_>), dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, ps, density_basis, xyz, \
+                       (uint64_t)M, out)
+    if (dtype == LM_F32) {
+        if (all64) LM_DX(float, 64); else LM_DX(float, 0);
+    } else {
+        if (all64) LM_DX(__half, 64); else LM_DX(__half, 0);
+    }
+#undef LM_DX
     LM_CHECK_LAUNCH("k_density_xyz");
     return LM_OK;
 }
