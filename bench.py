@@ -331,11 +331,20 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    copy_rate = None
     if args.calib:
         a = torch.ones(1 << 28, device="cuda:0")  # 1 GiB read + 1 GiB written by one copy kernel
         b = torch.empty_like(a)
         b.copy_(a)
         torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            b.copy_(a)
+        e1.record()
+        torch.cuda.synchronize()
+        copy_rate = 20 * 2 * a.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        log(f"[bench] device copy, 1 GiB: {copy_rate:.0f} GB/s (read + write)")
         del a, b
     if args.workload == "c2":
         out = bench_gather(args)
@@ -343,6 +352,8 @@ def main():
         out = bench_mlp(args)
     else:
         out = bench_frame(args, args.workload)
+    if copy_rate is not None:
+        out["hbm_copy_GBps"] = round(copy_rate, 1)
     print(json.dumps(out), flush=True)
 
 

@@ -147,6 +147,24 @@ int lm_relayout_nchw_to_hwc(const void *src, void *dst, int32_t C, int32_t H, in
 int lm_pack_occupancy(const float *vol, int32_t D, int32_t H, int32_t W, uint8_t *cells, uint32_t *not_binary,
                       void *stream);
 
+/* Alpha of a segment of length `length` at the gx*gy*gz lattice points
+ * aabb0*(1-s) + aabb1*s, s taken from the device tables lin_x[gx], lin_y[gy], lin_z[gz]
+ * (the caller's torch.linspace(0,1,g)): getDenseAlpha + compute_alpha
+ * (gridnerf_sequential.py:321-349, 401-427).  alpha is [gx][gy][gz] as the reference returns
+ * it.  If model->geom.vol is set it is the existing mask: points whose lookup is not > 0 keep
+ * sigma 0 (vol_thre is not used here).  Reads geom.aabb / inv_aabb / vol*, the density planes,
+ * density_basis, act, density_shift. */
+int lm_dense_alpha(const lm_model *model, const float *lin_x, const float *lin_y, const float *lin_z, int32_t gx,
+                   int32_t gy, int32_t gz, float length, float *alpha, void *stream);
+
+/* The pooling step of updateAlphaMask (gridnerf_sequential.py:351-384): clamp alpha
+ * [gx][gy][gz] to [0,1], transpose to [gz][gy][gx], 3x3x3 max pool (stride 1, padding 1),
+ * >= thres -> 1.0f else 0.0f into volume [gz][gy][gx].  box[6] (device int32) receives the
+ * smallest and largest x, y, z index of the voxels set (INT_MAX / -1 if none), count their
+ * number; the new AABB is the lattice coordinates at those indices. */
+int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, int32_t gz, float thres, float *volume,
+                       int32_t *box, uint64_t *count, void *stream);
+
 /* ---- part 1: sampling + AABB / occupancy culling + stable compaction -----------------
  * Replaces sample_ray / sample_ray_within_hull + AlphaGridMask.sample_alpha + the
  * boolean-mask indexing of GridBaseSequential.forward

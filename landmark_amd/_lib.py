@@ -56,6 +56,8 @@ SYMBOLS = {
     "lm_last_error": (C.c_char_p, []),
     "lm_relayout_nchw_to_hwc": (C.c_int, [_P, _P, _I32, _I32, _I32, _I32, _P]),
     "lm_pack_occupancy": (C.c_int, [_P, _I32, _I32, _I32, _P, _P, _P]),
+    "lm_dense_alpha": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _I32, _I32, _I32, _F, _P, _P]),
+    "lm_alpha_mask_pool": (C.c_int, [_P, _I32, _I32, _I32, _F, _P, _P, _P, _P]),
     "lm_sample_cull_scratch_bytes": (_SZ, [_I64, _I32]),
     "lm_sample_cull": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "lm_gather_density_xyz": (C.c_int, [C.POINTER(LmPlane), _I32, _P, _P, _I64, _P, _P]),

@@ -77,6 +77,7 @@ def params_from_checkpoint(
         alpha_volume=vol,
         alpha_aabb=aabb_m,
         alpha_mask_filter_thre=alpha_mask_filter_thre,
+        alphaMask_thres=float(kw.get("alphaMask_thres", 0.001)),
         encode_app="embedding_app.weight" in sd,
         embedding_app=sd.get("embedding_app.weight"),
         nonlinear_density="basis_den.weight" in sd,
@@ -106,7 +107,7 @@ def checkpoint_from_params(p: GridNeRFParams) -> dict:
     kwargs = {
         "aabb": p.aabb.cpu(), "gridSize": list(p.gridSize), "density_n_comp": n_ch(p.density_plane),
         "appearance_n_comp": n_ch(p.app_plane), "app_dim": p.app_dim, "density_shift": p.density_shift,
-        "alphaMask_thres": 0.001, "distance_scale": p.distance_scale, "rayMarch_weight_thres": p.rayMarch_weight_thres,
+        "alphaMask_thres": p.alphaMask_thres, "distance_scale": p.distance_scale, "rayMarch_weight_thres": p.rayMarch_weight_thres,
         "fea2denseAct": p.fea2denseAct, "near_far": list(p.near_far), "step_ratio": p.step_ratio, "pos_pe": 6,
         "view_pe": p.view_pe, "fea_pe": p.fea_pe, "featureC": p.featureC,
     }

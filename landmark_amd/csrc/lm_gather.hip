@@ -255,6 +255,41 @@ __global__ __launch_bounds__(kBlock) void k_app_xyz(PlaneSet ps, int K, const fl
     }
 }
 
+// ---- alpha on a lattice over the AABB (getDenseAlpha / compute_alpha) ------------------------
+// Point (i, j, k) = aabb0 * (1 - s) + aabb1 * s with s from three host tables, every product and
+// sum rounded on its own like the reference's tensor expression.  A point the existing occupancy
+// volume does not see (lookup not > 0) keeps sigma 0.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_dense_alpha(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
+                                                        const float *__restrict__ lin_x,
+                                                        const float *__restrict__ lin_y,
+                                                        const float *__restrict__ lin_z, int gx, int gy, int gz,
+                                                        int act, float shift, float length, float *__restrict__ alpha) {
+    const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
+    const uint64_t M = (uint64_t)gx * gy * gz;
+    const uint64_t n_tiles = (M + kTile - 1) / kTile;
+    for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
+        const uint64_t p = tile * kTile + slot;
+        if (p >= M) continue;
+        const int k = (int)(p % (uint64_t)gz), j = (int)((p / (uint64_t)gz) % (uint64_t)gy);
+        const int i = (int)(p / ((uint64_t)gz * gy));
+        const float s[3] = {lin_x[i], lin_y[j], lin_z[k]};
+        float pt[3], q[3];
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            const float a = g.aabb[d] * (1.0f - s[d]);
+            const float b = g.aabb[3 + d] * s[d];
+            pt[d] = a + b;
+        }
+        float sigma = 0.0f;
+        if (!g.vol || lm_alpha_lookup(g, pt) > 0.0f) {
+            lm_normalise(g, pt, q);
+            sigma = activate(density_sum<T>(ps, q, qlane, den_w), act, shift);
+        }
+        if (qlane == 0) alpha[p] = 1.0f - expf((-sigma) * length);
+    }
+}
+
 // ---- list driven (inside the render) -------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
@@ -641,6 +676,33 @@ extern "C" int lm_density_valid(const lm_model *m, const float *rays, const uint
         hipLaunchKernelGGL(k_density_list<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps,
                            m->density_basis, rays, valid_idx, counters + LM_STAT_N_VALID, m->act, m->density_shift, sigma);
     LM_CHECK_LAUNCH("k_density_list");
+    return LM_OK;
+}
+
+extern "C" int lm_dense_alpha(const lm_model *m, const float *lin_x, const float *lin_y, const float *lin_z,
+                              int32_t gx, int32_t gy, int32_t gz, float length, float *alpha, void *stream) {
+    LM_REQUIRE(m != nullptr, "model is null");
+    const lm_geom &g = m->geom;
+    if (g.vol) {
+        LM_REQUIRE(g.vd > 0 && g.vh > 0 && g.vw > 0, "occupancy volume has an empty dimension");
+        LM_REQUIRE(g.vol_dtype == LM_F32 || g.vol_dtype == LM_U8 || g.vol_dtype == LM_CELLS, "occupancy volume dtype %d",
+                   g.vol_dtype);
+    }
+    int dtype;
+    if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
+    LM_REQUIRE(gx > 0 && gy > 0 && gz > 0, "empty lattice %d x %d x %d", gx, gy, gz);
+    LM_REQUIRE(lin_x && lin_y && lin_z && alpha, "null buffer");
+    LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
+    const PlaneSet ps = make_set(m->density, m->n_planes);
+    const uint64_t tiles = ((uint64_t)gx * gy * gz + kTile - 1) / kTile;
+    const unsigned grid = (unsigned)std::min<uint64_t>(tiles, (uint64_t)lm_persistent_blocks(8));
+    if (dtype == LM_F32)
+        hipLaunchKernelGGL(k_dense_alpha<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, g, ps, m->density_basis,
+                           lin_x, lin_y, lin_z, gx, gy, gz, m->act, m->density_shift, length, alpha);
+    else
+        hipLaunchKernelGGL(k_dense_alpha<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, g, ps, m->density_basis,
+                           lin_x, lin_y, lin_z, gx, gy, gz, m->act, m->density_shift, length, alpha);
+    LM_CHECK_LAUNCH("k_dense_alpha");
     return LM_OK;
 }
 

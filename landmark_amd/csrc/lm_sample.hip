@@ -8,6 +8,8 @@
 //   k_emit         per-word prefix and the ascending list of valid flat indices
 // The list order is the row-major order of the reference's boolean-mask indexing
 // (app/models/gridnerf_sequential.py:461-465, 472), so indices match it exactly.
+#include <limits.h>
+
 #include "lm_common.h"
 
 namespace {
@@ -142,6 +144,57 @@ __global__ __launch_bounds__(256) void k_pack_occupancy(const float *__restrict_
     if (bad) *not_binary = 1u;  // plain store of the same value from every lane that sees one
 }
 
+// updateAlphaMask's pooling step: out[z][y][x] = 1 if the largest clamp(alpha, 0, 1) over the
+// 3 x 3 x 3 neighbourhood (cut at the borders) is >= thres, else 0; alpha is [gx][gy][gz].
+// box = {min x, y, z, max x, y, z} over the voxels set, count = their number.
+__global__ __launch_bounds__(256) void k_alpha_mask_pool(const float *__restrict__ alpha, int gx, int gy, int gz,
+                                                         float thres, float *__restrict__ out, int *__restrict__ box,
+                                                         unsigned long long *__restrict__ count) {
+    const size_t n = (size_t)gx * gy * gz;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    bool set = false;
+    int x = 0, y = 0, z = 0;
+    if (i < n) {
+        x = (int)(i % gx); y = (int)((i / gx) % gy); z = (int)(i / ((size_t)gx * gy));
+        float m = -INFINITY;
+        for (int dx = -1; dx <= 1; ++dx)
+            for (int dy = -1; dy <= 1; ++dy)
+                for (int dz = -1; dz <= 1; ++dz) {
+                    const int xx = x + dx, yy = y + dy, zz = z + dz;
+                    if (xx < 0 || xx >= gx || yy < 0 || yy >= gy || zz < 0 || zz >= gz) continue;
+                    float a = alpha[((size_t)xx * gy + yy) * gz + zz];
+                    a = fminf(fmaxf(a, 0.0f), 1.0f);
+                    m = fmaxf(m, a);
+                }
+        set = m >= thres;
+        out[i] = set ? 1.0f : 0.0f;
+    }
+    const uint64_t mask = __ballot(set);
+    if (mask == 0) return;
+    int lo[3] = {set ? x : INT_MAX, set ? y : INT_MAX, set ? z : INT_MAX};
+    int hi[3] = {set ? x : -1, set ? y : -1, set ? z : -1};
+    for (int off = 32; off > 0; off >>= 1)
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            lo[d] = min(lo[d], __shfl_xor(lo[d], off));
+            hi[d] = max(hi[d], __shfl_xor(hi[d], off));
+        }
+    if (lm_lane() == 0) {
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            atomicMin(box + d, lo[d]);
+            atomicMax(box + 3 + d, hi[d]);
+        }
+        atomicAdd(count, (unsigned long long)__popcll(mask));
+    }
+}
+
+__global__ void k_alpha_mask_init(int *box, unsigned long long *count) {
+    if (threadIdx.x < 3) box[threadIdx.x] = INT_MAX;
+    else if (threadIdx.x < 6) box[threadIdx.x] = -1;
+    else if (threadIdx.x == 6) *count = 0ull;
+}
+
 }  // namespace
 
 static uint64_t n_blocks_for(uint64_t n_words) { return (n_words + kWordsPerBlock - 1) / kWordsPerBlock; }
@@ -210,5 +263,19 @@ extern "C" int lm_pack_occupancy(const float *vol, int32_t D, int32_t H, int32_t
     hipLaunchKernelGGL(k_pack_occupancy, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, D, H, W,
                        cells, not_binary);
     LM_CHECK_LAUNCH("k_pack_occupancy");
+    return LM_OK;
+}
+
+extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, int32_t gz, float thres, float *volume,
+                                  int32_t *box, uint64_t *count, void *stream) {
+    LM_REQUIRE(alpha && volume && box && count, "null buffer");
+    LM_REQUIRE(gx > 0 && gy > 0 && gz > 0, "empty lattice %d x %d x %d", gx, gy, gz);
+    const size_t n = (size_t)gx * gy * gz;
+    LM_REQUIRE(n < ((size_t)1 << 39), "lattice too large");
+    hipLaunchKernelGGL(k_alpha_mask_init, dim3(1), dim3(64), 0, (hipStream_t)stream, box,
+                       reinterpret_cast<unsigned long long *>(count));
+    hipLaunchKernelGGL(k_alpha_mask_pool, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, alpha, gx,
+                       gy, gz, thres, volume, box, reinterpret_cast<unsigned long long *>(count));
+    LM_CHECK_LAUNCH("k_alpha_mask_pool");
     return LM_OK;
 }

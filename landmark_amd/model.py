@@ -69,26 +69,12 @@ class GridNeRFHIP:
         self.sampling_opt = params.sampling_opt
         self.ndims, self.resMode = params.ndims, list(params.resMode)
         self.nSamples = params.nSamples
-        self.alphaMask = None
-        if params.alpha_volume is not None:
-            vol = params.alpha_volume.to(self.device, torch.float32).contiguous()
-            self.alphaMask = SimpleNamespace(
-                alpha_volume=vol.view(1, 1, *vol.shape[-3:]), aabb=params.alpha_aabb.to(self.device)
-            )
-        self._vol = None if self.alphaMask is None else self.alphaMask.alpha_volume
-        self._vol_dtype, self._vol_store = L.LM_F32, self._vol
-        if self._vol is not None and occupancy in ("auto", "cells", "u8"):
-            D, H, W = self._vol.shape[-3:]
-            cells = torch.empty((D + 1) * (H + 1) * (W + 1), dtype=torch.uint8, device=self.device)
-            flag = torch.zeros(1, dtype=torch.int32, device=self.device)
-            L.check(self.lib.lm_pack_occupancy(self._vol.data_ptr(), D, H, W, cells.data_ptr(), flag.data_ptr(), L.current_stream()), "lm_pack_occupancy")
-            if occupancy != "u8" and int(flag.item()) == 0:
-                # a 0/1 mask (what the reference stores): one byte per trilinear cell, one load per sample
-                self._vol_dtype, self._vol_store = L.LM_CELLS, cells
-            else:
-                as_u8 = self._vol.clamp(0, 255).to(torch.uint8)
-                if bool((as_u8.float() == self._vol).all()):
-                    self._vol_dtype, self._vol_store = L.LM_U8, as_u8.contiguous()
+        self.alphaMask_thres = params.alphaMask_thres
+        self.gridSize = list(params.gridSize)
+        self.stepSize = params.stepSize
+        self._occupancy = occupancy
+        self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
+        self._set_alpha_mask(params.alpha_volume, params.alpha_aabb)
         # --- channel-last tables
         self._tables = []  # keep device tensors alive
         self._density = self._relayout_set(params.density_plane, params.density_line)
@@ -114,12 +100,35 @@ class GridNeRFHIP:
         self._packed = {}
         self._bias_code = {}
         self._pack_mlp(mlp_precision)
-        # --- per-S geometry and workspace caches
-        self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
+        # --- workspace cache (per-S geometry is cached in _geom_cache)
         self._ws = None
         self.counters = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------------ construction helpers
+    def _set_alpha_mask(self, volume, aabb):
+        """Install an occupancy volume [D,H,W] (AlphaGridMask, app/models/alpha_mask.py:16-26) or none."""
+        self._geom_cache.clear()
+        self.alphaMask = None
+        self._vol, self._vol_store, self._vol_dtype, self._alpha_aabb = None, None, L.LM_F32, None
+        if volume is None:
+            return
+        vol = volume.to(self.device, torch.float32).contiguous()
+        self._alpha_aabb = aabb.detach().to(torch.float32).cpu()
+        self.alphaMask = SimpleNamespace(alpha_volume=vol.view(1, 1, *vol.shape[-3:]), aabb=aabb.to(self.device))
+        self._vol = self._vol_store = self.alphaMask.alpha_volume
+        if self._occupancy in ("auto", "cells", "u8"):
+            D, H, W = self._vol.shape[-3:]
+            cells = torch.empty((D + 1) * (H + 1) * (W + 1), dtype=torch.uint8, device=self.device)
+            flag = torch.zeros(1, dtype=torch.int32, device=self.device)
+            L.check(self.lib.lm_pack_occupancy(self._vol.data_ptr(), D, H, W, cells.data_ptr(), flag.data_ptr(), L.current_stream()), "lm_pack_occupancy")
+            if self._occupancy != "u8" and int(flag.item()) == 0:
+                # a 0/1 mask (what the reference stores): one byte per trilinear cell, one load per sample
+                self._vol_dtype, self._vol_store = L.LM_CELLS, cells
+            else:
+                as_u8 = self._vol.clamp(0, 255).to(torch.uint8)
+                if bool((as_u8.float() == self._vol).all()):
+                    self._vol_dtype, self._vol_store = L.LM_U8, as_u8.contiguous()
+
     def _relayout(self, t: torch.Tensor) -> torch.Tensor:
         """[1,C,H,W] -> device [H,W,C] through lm_relayout_nchw_to_hwc."""
         src = t.to(self.device).contiguous()
@@ -223,7 +232,7 @@ class GridNeRFHIP:
             g.vol = self._vol_store.data_ptr()
             g.vol_dtype = self._vol_dtype
             g.vd, g.vh, g.vw = self._vol.shape[-3:]
-            ab = p.alpha_aabb.detach().cpu()
+            ab = self._alpha_aabb
             g.vol_aabb_min[:] = ab[0].tolist()
             g.vol_inv[:] = (1.0 / (ab[1] - ab[0]) * 2).tolist()
             g.vol_thre = torch.tensor(p.alpha_mask_filter_thre, dtype=torch.float32).item()
@@ -312,6 +321,53 @@ class GridNeRFHIP:
             ),
             "lm_render",
         )
+
+    # ------------------------------------------------------------------ occupancy volume from the model
+    @torch.no_grad()
+    def getDenseAlpha(self, gridSize=None):
+        """Alpha of one step at the lattice points of the AABB -> (alpha [gx,gy,gz], dense_xyz [gx,gy,gz,3])
+        (gridnerf_sequential.py:321-349)."""
+        gs = [int(v) for v in (self.gridSize if gridSize is None else gridSize)]
+        lin = [torch.linspace(0, 1, g).to(self.device) for g in gs]
+        samples = torch.stack(torch.meshgrid(*lin, indexing="ij"), -1)
+        dense_xyz = self.aabb[0] * (1 - samples) + self.aabb[1] * samples
+        alpha = torch.empty(gs, dtype=torch.float32, device=self.device)
+        m = self._model_struct(self._samples_for(-1), True)
+        length = torch.as_tensor(self.stepSize, dtype=torch.float32).item()
+        L.check(
+            self.lib.lm_dense_alpha(C.byref(m), lin[0].data_ptr(), lin[1].data_ptr(), lin[2].data_ptr(), gs[0], gs[1], gs[2],
+                                    length, alpha.data_ptr(), L.current_stream()),
+            "lm_dense_alpha",
+        )
+        torch.cuda.current_stream().synchronize()  # the tables are temporaries
+        return alpha, dense_xyz
+
+    @torch.no_grad()
+    def updateAlphaMask(self, gridSize=(200, 200, 200), increase_alpha_thresh=0):
+        """Rebuild the occupancy volume from the density field and return the tight AABB of what is occupied
+        (gridnerf_sequential.py:351-384)."""
+        gs = [int(v) for v in gridSize]
+        alpha, _ = self.getDenseAlpha(gs)
+        thres = torch.tensor(self.alphaMask_thres * (10**increase_alpha_thresh), dtype=torch.float32).item()
+        volume = torch.empty(gs[::-1], dtype=torch.float32, device=self.device)
+        box = torch.empty(6, dtype=torch.int32, device=self.device)
+        count = torch.empty(1, dtype=torch.int64, device=self.device)
+        L.check(
+            self.lib.lm_alpha_mask_pool(alpha.data_ptr(), gs[0], gs[1], gs[2], thres, volume.data_ptr(), box.data_ptr(),
+                                        count.data_ptr(), L.current_stream()),
+            "lm_alpha_mask_pool",
+        )
+        self._set_alpha_mask(volume, self.aabb)
+        b = box.cpu().tolist()
+        if int(count.item()) == 0:
+            raise L.LandmarkError("updateAlphaMask: no voxel reaches the threshold")
+        a0, a1 = self.aabb[0].cpu(), self.aabb[1].cpu()
+        lin = [torch.linspace(0, 1, g) for g in gs]
+        lo = torch.stack([a0[d] * (1 - lin[d][b[d]]) + a1[d] * lin[d][b[d]] for d in range(3)])
+        hi = torch.stack([a0[d] * (1 - lin[d][b[3 + d]]) + a1[d] * lin[d][b[3 + d]] for d in range(3)])
+        total = gs[0] * gs[1] * gs[2]
+        self.alpha_rest_percent = int(count.item()) / total * 100
+        return torch.stack((lo, hi)).to(self.device)
 
     def last_counts(self) -> Dict[str, int]:
         """Valid / appearance sample counts of the last chunk (synchronises)."""

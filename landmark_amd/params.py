@@ -47,6 +47,7 @@ class GridNeRFParams:
     alpha_volume: Optional[torch.Tensor] = None  # [D,H,W] float {0,1}
     alpha_aabb: Optional[torch.Tensor] = None  # [2,3]
     alpha_mask_filter_thre: float = 0.0
+    alphaMask_thres: float = 0.001  # threshold updateAlphaMask applies (gridnerf_sequential.py:57, 366-367)
     # per-image appearance embedding (args.encode_app, gridnerf_sequential.py:681-682): the
     # first Linear then takes 27 + 48 + 3 + 108 + 12 = 198 inputs (mlp_render_fea.py:23-24)
     encode_app: bool = False
@@ -110,6 +111,7 @@ class GridNeRFParams:
             alpha_volume=mv(self.alpha_volume),
             alpha_aabb=mv(self.alpha_aabb),
             alpha_mask_filter_thre=self.alpha_mask_filter_thre,
+            alphaMask_thres=self.alphaMask_thres,
             encode_app=self.encode_app,
             embedding_app=mv(self.embedding_app),
             nonlinear_density=self.nonlinear_density,

@@ -20,6 +20,8 @@ How each function is pinned (tests/test_oracle_*.py):
   raw2alpha                                  double-loop volume rendering, closed forms
   positional_encoding                        math.sin / math.cos, index order
   mlp_render                                 fp64 numpy matmul chain
+  compute_alpha / get_dense_alpha /          golden vectors (tests/golden/alphamask_*.npz) written from
+  update_alpha_mask                          the reference's getDenseAlpha / updateAlphaMask
   render_chunk (composition order)           golden vectors written by
                                              tests/golden/make_golden.py from the
                                              reference's own forward
@@ -158,6 +160,46 @@ def feature2density(p, f):
     if p.fea2denseAct == "relu":
         return F.relu(f)
     raise ValueError(p.fea2denseAct)
+
+
+# --------------------------------------------------------------------------------------
+# occupancy volume from the density field
+# --------------------------------------------------------------------------------------
+def compute_alpha(p, xyz_locs, length):
+    """Alpha of a segment of `length` at world points [M,3], gridnerf_sequential.py:401-427."""
+    if p.alpha_volume is not None:
+        on = sample_alpha(p.alpha_volume, p.alpha_aabb, xyz_locs) > 0
+    else:
+        on = torch.ones_like(xyz_locs[:, 0], dtype=torch.bool)
+    sigma = torch.zeros(xyz_locs.shape[:-1])
+    if on.any():
+        sigma[on] = feature2density(p, density_feature(p, normalize_coord(p, xyz_locs[on])))
+    return 1 - torch.exp(-sigma * length)
+
+
+def get_dense_alpha(p, gridSize=None):
+    """(alpha [gx,gy,gz], dense_xyz [gx,gy,gz,3]) on the lattice of the AABB, gridnerf_sequential.py:321-349."""
+    gs = list(p.gridSize if gridSize is None else gridSize)
+    samples = torch.stack(torch.meshgrid(*[torch.linspace(0, 1, g) for g in gs], indexing="ij"), -1)
+    dense_xyz = p.aabb[0] * (1 - samples) + p.aabb[1] * samples
+    alpha = torch.zeros_like(dense_xyz[..., 0])
+    for i in range(gs[0]):
+        alpha[i] = compute_alpha(p, dense_xyz[i].view(-1, 3), p.stepSize).view(gs[1], gs[2])
+    return alpha, dense_xyz
+
+
+def update_alpha_mask(p, gridSize=(200, 200, 200), increase_alpha_thresh=0):
+    """(new_aabb [2,3], volume [gz,gy,gx]) of gridnerf_sequential.py:351-384; the new mask's box is p.aabb."""
+    gs = list(gridSize)
+    alpha, dense_xyz = get_dense_alpha(p, gs)
+    dense_xyz = dense_xyz.transpose(0, 2).contiguous()
+    alpha = alpha.clamp(0, 1).transpose(0, 2).contiguous()[None, None]
+    alpha = F.max_pool3d(alpha, kernel_size=3, padding=1, stride=1).view(gs[::-1])
+    thres = p.alphaMask_thres * (10**increase_alpha_thresh)
+    alpha[alpha >= thres] = 1
+    alpha[alpha < thres] = 0
+    valid = dense_xyz[alpha > 0.5]
+    return torch.stack((valid.amin(0), valid.amax(0))), alpha
 
 
 # --------------------------------------------------------------------------------------

@@ -206,5 +206,79 @@ def main():
               f"weights>thr {n_app} rgb mean {out['rgb_map'].mean():.4f} -> {os.path.getsize(path)/1024:.0f} KB")
 
 
+ALPHA_CASES = [
+    # the occupancy volume rebuilt from the density field (getDenseAlpha + updateAlphaMask)
+    dict(name="softplus_nomask", grid=[6, 7, 5], act="softplus", shift=-10.0, res=[1], ndims=3, mask=False, boost=150.0, gs=(13, 11, 9), inc=0),
+    dict(name="relu_L2_mask_inc1", grid=[6, 7, 5], act="relu", shift=-10.0, res=[1, 2], ndims=3, mask=True, boost=6.0, gs=(10, 14, 12), inc=1),
+]
+
+
+def main_alpha():
+    """Fixtures alphamask_*.npz: getDenseAlpha on the model's own grid and updateAlphaMask on another."""
+    _install_stand_ins()
+    sys.path.insert(0, REF)
+    from app.models.alpha_mask import AlphaGridMask  # noqa: E402
+    from app.models.gridnerf_sequential import GridNeRF  # noqa: E402
+
+    for ci, c in enumerate(ALPHA_CASES):
+        torch.manual_seed(300 + ci)
+        aabb = torch.tensor([[-1.0, -1.2, -0.8], [1.1, 1.0, 0.9]])
+        args = _args(ndims=c["ndims"], resMode=c["res"], sampling_opt=1, n_importance=16)
+        model = GridNeRF(
+            aabb, c["grid"], "cpu",
+            density_n_comp=[16] * 3, appearance_n_comp=[48] * 3, app_dim=27,
+            near_far=[0.4, 4.0], density_shift=c["shift"], distance_scale=25, rayMarch_weight_thres=0.001,
+            pos_pe=2, view_pe=2, fea_pe=2, featureC=128, step_ratio=2.0,
+            fea2denseAct=c["act"], args=args, is_train=False,
+        )
+        model.eval()
+        with torch.no_grad():
+            # density only inside an off-centre box (normalised coordinates), so that the rebuilt volume
+            # has empty borders of different widths on every axis
+            lo, hi = (-0.1, -0.7, -0.45), (0.75, 0.2, 0.35)
+            for k, (pl, ln) in enumerate(zip(model.density_plane, model.density_line)):
+                d = k // len(c["res"])
+                m0, m1 = [[0, 1], [0, 2], [1, 2]][d]
+                v = [2, 1, 0][d]
+                pl.mul_(c["boost"])
+                cw = torch.linspace(-1, 1, pl.shape[3])
+                ch = torch.linspace(-1, 1, pl.shape[2])
+                pl.mul_(((cw >= lo[m0]) & (cw <= hi[m0])).float()[None, None, None, :])
+                pl.mul_(((ch >= lo[m1]) & (ch <= hi[m1])).float()[None, None, :, None])
+                cl = torch.linspace(-1, 1, ln.shape[2])
+                ln.mul_(((cl >= lo[v]) & (cl <= hi[v])).float()[None, None, :, None])
+            store = {"aabb": aabb}
+            if c["mask"]:
+                g = torch.Generator().manual_seed(40 + ci)
+                vol = (torch.rand(5, 7, 6, generator=g) < 0.7).float()
+                mask_aabb = aabb + torch.tensor([[0.05, -0.02, 0.0], [0.0, 0.03, -0.04]])
+                model.alphaMask = AlphaGridMask("cpu", mask_aabb, vol)
+                store["alpha_volume"], store["alpha_aabb"] = vol, mask_aabb
+            for k, v in model.state_dict().items():
+                store["sd." + k] = v
+            alpha, dense_xyz = model.getDenseAlpha()
+            store["dense_alpha"], store["dense_xyz"] = alpha, dense_xyz
+            alpha2, _ = model.getDenseAlpha(c["gs"])
+            store["dense_alpha_gs"] = alpha2
+            new_aabb = model.updateAlphaMask(c["gs"], increase_alpha_thresh=c["inc"])
+            store["new_aabb"] = new_aabb
+            store["new_volume"] = model.alphaMask.alpha_volume[0, 0]
+            store["new_mask_aabb"] = model.alphaMask.aabb
+        cfg = dict(
+            grid=c["grid"], ndims=c["ndims"], resMode=c["res"], near_far=[0.4, 4.0], density_shift=c["shift"],
+            fea2denseAct=c["act"], step_ratio=2.0, stepSize=float(model.stepSize), gs=list(c["gs"]), inc=c["inc"],
+            alphaMask_thres=float(model.alphaMask_thres),
+        )
+        arrays = {k: (v.detach().cpu().numpy() if torch.is_tensor(v) else np.asarray(v)) for k, v in store.items()}
+        arrays["cfg_json"] = np.frombuffer(__import__("json").dumps(cfg).encode(), dtype=np.uint8)
+        path = os.path.join(HERE, f"alphamask_{c['name']}.npz")
+        np.savez_compressed(path, **arrays)
+        a = arrays["dense_alpha_gs"]
+        print(f"alphamask_{c['name']}: alpha range [{a.min():.2e}, {a.max():.2e}] occupied {int(arrays['new_volume'].sum())}/"
+              f"{arrays['new_volume'].size} new_aabb {arrays['new_aabb'].tolist()} -> {os.path.getsize(path)/1024:.0f} KB")
+
+
 if __name__ == "__main__":
-    main()
+    if "--alpha-only" not in sys.argv:
+        main()
+    main_alpha()

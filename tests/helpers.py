@@ -15,9 +15,13 @@ def golden_names():
     return sorted(os.path.basename(p)[len("forward_") : -len(".npz")] for p in glob.glob(os.path.join(GOLDEN_DIR, "forward_*.npz")))
 
 
-def load_golden(name):
+def alphamask_names():
+    return sorted(os.path.basename(p)[len("alphamask_") : -len(".npz")] for p in glob.glob(os.path.join(GOLDEN_DIR, "alphamask_*.npz")))
+
+
+def load_golden(name, kind="forward"):
     """(params, data dict of tensors, cfg) for one fixture written by golden/make_golden.py."""
-    z = np.load(os.path.join(GOLDEN_DIR, f"forward_{name}.npz"))
+    z = np.load(os.path.join(GOLDEN_DIR, f"{kind}_{name}.npz"))
     cfg = json.loads(bytes(z["cfg_json"]).decode())
     data = {k: torch.from_numpy(z[k]) for k in z.files if k != "cfg_json"}
     n = cfg["ndims"] * len(cfg["resMode"])
@@ -41,11 +45,12 @@ def load_golden(name):
         rayMarch_weight_thres=1e-3,
         fea2denseAct=cfg["fea2denseAct"],
         step_ratio=cfg["step_ratio"],
-        sampling_opt=cfg["sampling_opt"],
-        n_importance=cfg["n_importance"],
+        sampling_opt=cfg.get("sampling_opt", 1),
+        n_importance=cfg.get("n_importance", 16),
         alpha_volume=data.get("alpha_volume"),
         alpha_aabb=data.get("alpha_aabb"),
-        alpha_mask_filter_thre=cfg["thre"],
+        alpha_mask_filter_thre=cfg.get("thre", 0.0),
+        alphaMask_thres=cfg.get("alphaMask_thres", 0.001),
         encode_app=cfg.get("encode_app", False),
         embedding_app=sd.get("embedding_app.weight"),
         nonlinear_density=cfg.get("nonlinear_density", False),

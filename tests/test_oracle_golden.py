@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import gridnerf_oracle as O
-from tests.helpers import golden_names, load_golden
+from tests.helpers import alphamask_names, golden_names, load_golden
 
 NAMES = golden_names()
 
@@ -64,3 +64,46 @@ def test_chunk_driver_is_chunk_invariant():
         # colour network may differ in the last bits between chunkings
         assert torch.allclose(ret["rgb_map"], full["rgb_map"], atol=1e-6, rtol=0)
         assert torch.equal(ret["depth_map"], full["depth_map"])
+
+
+@pytest.mark.parametrize("name", alphamask_names())
+def test_alpha_mask_update_matches_reference(name):
+    """getDenseAlpha / updateAlphaMask of the reference (tests/golden/alphamask_*.npz)."""
+    p, d, cfg = load_golden(name, kind="alphamask")
+    assert float(p.stepSize) == pytest.approx(cfg["stepSize"], rel=1e-6)
+    alpha, xyz = O.get_dense_alpha(p)
+    assert torch.equal(xyz, d["dense_xyz"]) and torch.equal(alpha, d["dense_alpha"])
+    alpha_gs, _ = O.get_dense_alpha(p, cfg["gs"])
+    assert torch.equal(alpha_gs, d["dense_alpha_gs"])
+    new_aabb, vol = O.update_alpha_mask(p, cfg["gs"], cfg["inc"])
+    assert torch.equal(vol, d["new_volume"]) and torch.equal(new_aabb, d["new_aabb"])
+    assert torch.equal(d["new_mask_aabb"], p.aabb)
+    # the fixture is discriminating: some but not all voxels are set, and the box is tight on every axis
+    assert 0 < int(vol.sum()) < vol.numel()
+    assert bool((new_aabb[0] > p.aabb[0]).any()) and bool((new_aabb[1] < p.aabb[1]).any())
+
+
+def test_alpha_mask_pool_brute_force():
+    """update_alpha_mask's pooling against a plain triple loop on a random lattice."""
+    p, d, cfg = load_golden(alphamask_names()[0], kind="alphamask")
+    gs = [5, 4, 6]
+    alpha, xyz = O.get_dense_alpha(p, gs)
+    new_aabb, vol = O.update_alpha_mask(p, gs, 0)
+    a = alpha.clamp(0, 1)
+    lo, hi = [None] * 3, [None] * 3
+    for x in range(gs[0]):
+        for y in range(gs[1]):
+            for z in range(gs[2]):
+                m = max(
+                    float(a[xx, yy, zz])
+                    for xx in range(max(x - 1, 0), min(x + 2, gs[0]))
+                    for yy in range(max(y - 1, 0), min(y + 2, gs[1]))
+                    for zz in range(max(z - 1, 0), min(z + 2, gs[2]))
+                )
+                want = 1.0 if m >= p.alphaMask_thres else 0.0
+                assert float(vol[z, y, x]) == want
+                if want:
+                    for k, v in enumerate(xyz[x, y, z].tolist()):
+                        lo[k] = v if lo[k] is None else min(lo[k], v)
+                        hi[k] = v if hi[k] is None else max(hi[k], v)
+    assert new_aabb[0].tolist() == lo and new_aabb[1].tolist() == hi
