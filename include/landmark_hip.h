@@ -90,6 +90,16 @@ typedef struct lm_geom {
     float vol_aabb_min[3];
     float vol_inv[3];
     float vol_thre; /* alpha_mask_filter_thre */
+    /* Block-stacked model (the "-merged-stack" checkpoint, gridnerf_branch_parallel.py:465-527,
+     * rendered through assign_blocks_to_samples, gridnerf_parallel.py:279-338): the XY extent is
+     * cut into div0 x div1 blocks, block b = floor((x+1)/blk_w)*div1 + floor((y+1)/blk_h) of the
+     * normalised sample, planes are [B][H][W][C] and lines [Len][B][C] with B = div0*div1, H, W
+     * the size of one block, and x, y are re-normalised to the block before the lookup.
+     * blk_w = (float)(2.0/div0), blk_h = (float)(2.0/div1).  div0 == 0: one block, plain tables.
+     * The reference interpolates over the block axis with a block coordinate that is an integer
+     * up to float rounding; here the lookup reads block b alone (difference below 1e-6 relative). */
+    int32_t div0, div1;
+    float blk_w, blk_h;
 } lm_geom;
 
 /* stages of lm_render, in launch order */

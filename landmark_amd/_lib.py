@@ -36,6 +36,7 @@ class LmGeom(C.Structure):
         ("tab_a", C.c_void_p), ("tab_t", C.c_void_p), ("inv_aabb", C.c_float * 3),
         ("vol", C.c_void_p), ("vd", C.c_int32), ("vh", C.c_int32), ("vw", C.c_int32), ("vol_dtype", C.c_int32),
         ("vol_aabb_min", C.c_float * 3), ("vol_inv", C.c_float * 3), ("vol_thre", C.c_float),
+        ("div0", C.c_int32), ("div1", C.c_int32), ("blk_w", C.c_float), ("blk_h", C.c_float),
     ]
 
 

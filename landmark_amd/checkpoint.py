@@ -8,7 +8,10 @@ k = dim * len(resMode) + level; basis_mat.weight; renderModule.mlp.{0,2,4}.{weig
 optional basis_den.weight (nonlinear_density) and embedding_app.weight (encode_app).
 What is not stored in the file (ndims / resMode split of the plane count, sampler choice,
 n_importance, alpha_mask_filter_thre) comes from the run configuration and is passed in.
-The block-stacked "-merged-stack" layout of the parallel trainers is not handled here.
+The block-stacked "-merged-stack" layout of the branch-parallel trainer
+(app/models/gridnerf_branch_parallel.py:465-527: planes [1,C,B,h,w], lines [1,C,L,B], B =
+plane_division[0] * plane_division[1], kwargs["args"] = the run's arguments as a dict) is read
+too; plane_division comes from that dict or from the caller.
 """
 from __future__ import annotations
 
@@ -28,8 +31,10 @@ def params_from_checkpoint(
     n_importance: int = 128,
     alpha_mask_filter_thre: float = 0.0,
     near_far: Optional[Sequence[float]] = None,
+    plane_division: Optional[Sequence[int]] = None,
 ) -> GridNeRFParams:
     kw, sd = ckpt["kwargs"], ckpt["state_dict"]
+    sd = {k.replace(".module", "").replace(".params", ""): v for k, v in sd.items()}  # DDP / wrapper prefixes
     n = len([k for k in sd if k.startswith("density_plane.")])
     if n == 0:
         raise ValueError("checkpoint holds no density_plane.* tensors (a stacked multi-block checkpoint?)")
@@ -40,9 +45,19 @@ def params_from_checkpoint(
         ndims = n // len(resMode)
     if ndims * len(resMode) != n:
         raise ValueError(f"ndims {ndims} x levels {len(resMode)} != {n} planes in the checkpoint")
-    for k in range(n):
-        if sd[f"density_plane.{k}"].dim() != 4:
-            raise ValueError("block-stacked planes ([1,C,B,h,w]) are not supported by this loader")
+    stacked = sd["density_plane.0"].dim() == 5  # "-merged-stack" layout, gridnerf_branch_parallel.py:465-527
+    if stacked:
+        if plane_division is None:
+            saved = kw.get("args")
+            plane_division = saved.get("plane_division") if isinstance(saved, dict) else None
+        if plane_division is None:
+            raise ValueError("block-stacked planes ([1,C,B,h,w]): plane_division is needed")
+        B = int(plane_division[0]) * int(plane_division[1])
+        for k in range(n):
+            if sd[f"density_plane.{k}"].dim() != 5 or sd[f"density_plane.{k}"].shape[2] != B or sd[f"density_line.{k}"].shape[-1] != B:
+                raise ValueError(f"plane {k} does not hold {B} blocks")
+    else:
+        plane_division = None
     has_bias = "renderModule.mlp.0.bias" in sd
     vol = aabb_m = None
     if "alphaMask.aabb" in ckpt:
@@ -82,6 +97,7 @@ def params_from_checkpoint(
         embedding_app=sd.get("embedding_app.weight"),
         nonlinear_density="basis_den.weight" in sd,
         basis_den=sd.get("basis_den.weight"),
+        plane_division=None if plane_division is None else [int(v) for v in plane_division],
     )
 
 
@@ -111,6 +127,8 @@ def checkpoint_from_params(p: GridNeRFParams) -> dict:
         "fea2denseAct": p.fea2denseAct, "near_far": list(p.near_far), "step_ratio": p.step_ratio, "pos_pe": 6,
         "view_pe": p.view_pe, "fea_pe": p.fea_pe, "featureC": p.featureC,
     }
+    if p.plane_division is not None:
+        kwargs["args"] = {"plane_division": list(p.plane_division)}
     ckpt = {"kwargs": kwargs, "state_dict": sd}
     if p.alpha_volume is not None:
         vol = p.alpha_volume.bool().cpu().numpy()

@@ -152,6 +152,11 @@ int check_model(const lm_model *m, int *K) {
     int dt;
     if (int rc = lm_check_planes(m->density, m->n_planes, &dt, nullptr)) return rc;
     if (int rc = lm_check_planes(m->app, m->n_planes, &dt, K)) return rc;
+    if (m->geom.div0 > 0)
+        for (int k = 0; k < m->n_planes; ++k)
+            for (const lm_plane *pl : {&m->density[k], &m->app[k]})
+                LM_REQUIRE(pl->ax0 == 0 && pl->ax1 == 1 && pl->axl == 2,
+                           "a block-stacked model has XY planes and z lines only (plane %d)", k);
     return LM_OK;
 }
 }  // namespace

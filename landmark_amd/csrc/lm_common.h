@@ -97,6 +97,44 @@ __device__ __forceinline__ void lm_normalise(const lm_geom &g, const float *pt, 
     }
 }
 
+// Block of a block-stacked model and the coordinates inside it, with the reference's float
+// operations (assign_blocks_to_samples, app/models/gridnerf_parallel.py:300-328; floor_divide and
+// remainder as ATen defines them for floats).  q[0], q[1] are replaced; returns the block index.
+__device__ __forceinline__ float lm_floor_divide(float a, float b) {
+    const float mod = fmodf(a, b);
+    float div = (a - mod) / b;
+    if (mod != 0.0f && ((b < 0.0f) != (mod < 0.0f))) div = div - 1.0f;
+    if (div == 0.0f) return copysignf(0.0f, a / b);
+    float fl = floorf(div);
+    if (div - fl > 0.5f) fl = fl + 1.0f;
+    return fl;
+}
+__device__ __forceinline__ float lm_remainder(float a, float b) {
+    float mod = fmodf(a, b);
+    if (mod != 0.0f && ((b < 0.0f) != (mod < 0.0f))) mod = mod + b;
+    return mod;
+}
+__device__ __forceinline__ int lm_block_coords(const lm_geom &g, float *q) {
+    const float d1 = (float)g.div1;
+    const float xs = (q[0] + 1.0f) / g.blk_w, ys = (q[1] + 1.0f) / g.blk_h;
+    const float fx = floorf(xs) * d1;
+    const float b = fx + floorf(ys);
+    const float bx = lm_floor_divide(b, d1), by = lm_remainder(b, d1);
+    const float sz[2] = {g.blk_w, g.blk_h}, bi[2] = {bx, by};
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const float m0 = bi[k] * sz[k];
+        const float lo = -1.0f + m0;
+        const float m1 = (bi[k] + 1.0f) * sz[k];
+        const float hi = -1.0f + m1;
+        const float t = (q[k] - lo) * 2.0f;
+        const float u = t / (hi - lo);
+        q[k] = u - 1.0f;
+    }
+    // b is integer valued; the clamp keeps the conversion defined for far-away points
+    return (int)fminf(fmaxf(b, -1.0f), 1.0e9f);
+}
+
 // Trilinear lookup with zero padding and align_corners=True in ATen's operation order
 // (corner order tnw, tne, tsw, tse, bnw, bne, bsw, bse; weight = (x)(y)(z) left to right;
 // each value*weight rounded before it is added).

@@ -26,6 +26,7 @@ constexpr int kTile = kBlock / kQuad;  // samples per workgroup iteration
 struct PlaneSet {
     lm_plane p[LM_MAX_PLANES];
     int n;
+    int nblk;  // > 0: block-stacked tables, planes [nblk][H][W][C], lines [Len][nblk][C]
 };
 
 template <typename T> struct Vec;
@@ -95,6 +96,22 @@ __device__ __forceinline__ Taps1 line_taps(const lm_plane &pl, float c) {
     return t;
 }
 
+// Queries are float[4]: normalised x, y, z and, for block-stacked tables, the block index as
+// integer bits in q[3].  Moves the taps to the block; a block outside the table reads as zero.
+__device__ __forceinline__ void block_taps(const lm_plane &pl, int nblk, const float *q, Taps2 &t2, Taps1 &t1) {
+    if (nblk <= 0) return;
+    const int blk = __float_as_int(q[3]);
+    if (blk < 0 || blk >= nblk) {
+        t2.w00 = t2.w01 = t2.w10 = t2.w11 = 0.0f;
+        t1.w0 = t1.w1 = 0.0f;
+        return;
+    }
+    const int64_t base = (int64_t)blk * pl.H * pl.W * pl.C;
+    t2.o00 += base; t2.o01 += base; t2.o10 += base; t2.o11 += base;
+    t1.o0 = t1.o0 * nblk + blk * pl.C;
+    t1.o1 = t1.o1 * nblk + blk * pl.C;
+}
+
 __device__ __forceinline__ float pick(const float *q, int ax) { return ax == 0 ? q[0] : (ax == 1 ? q[1] : q[2]); }
 
 // products of one plane for the V channels starting at c (lane-private)
@@ -131,8 +148,9 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
         const lm_plane &pl = ps.p[k];
-        const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-        const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+        Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        block_taps(pl, ps.nblk, q, t2, t1);
         for (int c = V * qlane; c < pl.C; c += V * kQuad) {
             float prod[V];
             plane_products<T>(pl, t2, t1, c, prod);
@@ -162,8 +180,9 @@ __device__ __forceinline__ float density_sum_fixed(const PlaneSet &ps, const flo
     float sum = 0.0f;
     for (int k = 0; k < ps.n; ++k) {
         const lm_plane &pl = ps.p[k];
-        const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-        const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+        Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        block_taps(pl, ps.nblk, q, t2, t1);
         float prod[NG][V];
 #pragma unroll
         for (int gi = 0; gi < NG; ++gi) {
@@ -190,8 +209,9 @@ __device__ __forceinline__ void app_store(const PlaneSet &ps, const float *q, un
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
         const lm_plane &pl = ps.p[k];
-        const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-        const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+        Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+        block_taps(pl, ps.nblk, q, t2, t1);
         for (int c = V * qlane; c < pl.C; c += V * kQuad) {
             float prod[V];
             plane_products<T>(pl, t2, t1, c, prod);
@@ -215,6 +235,7 @@ __device__ __forceinline__ void list_coords(const lm_geom &g, const float *__res
     float pt[3];
     lm_point(ray, z, pt);
     lm_normalise(g, pt, q);
+    q[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q) : 0);
 }
 
 __device__ __forceinline__ float activate(float f, int act, float shift) {
@@ -235,7 +256,7 @@ __global__ __launch_bounds__(kBlock) void k_density_xyz(PlaneSet ps, const float
     for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
         const uint64_t p = tile * kTile + slot;
         if (p >= M) continue;
-        float q[3] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2]};
+        float q[4] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2], 0.0f};
         const float s = CFIX > 0 ? density_sum_fixed<T, (CFIX > 0 ? CFIX : 16)>(ps, q, qlane, den_w)
                                  : density_sum<T>(ps, q, qlane, den_w);
         if (qlane == 0) out[p] = s;
@@ -250,7 +271,7 @@ __global__ __launch_bounds__(kBlock) void k_app_xyz(PlaneSet ps, int K, const fl
     for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
         const uint64_t p = tile * kTile + slot;
         if (p >= M) continue;
-        float q[3] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2]};
+        float q[4] = {xyz[3 * p], xyz[3 * p + 1], xyz[3 * p + 2], 0.0f};
         app_store<T>(ps, q, qlane, out + p * (uint64_t)K);
     }
 }
@@ -274,7 +295,8 @@ __global__ __launch_bounds__(kBlock) void k_dense_alpha(lm_geom g, PlaneSet ps, 
         const int k = (int)(p % (uint64_t)gz), j = (int)((p / (uint64_t)gz) % (uint64_t)gy);
         const int i = (int)(p / ((uint64_t)gz * gy));
         const float s[3] = {lin_x[i], lin_y[j], lin_z[k]};
-        float pt[3], q[3];
+        float pt[3], q[4];
+        q[3] = 0.0f;
 #pragma unroll
         for (int d = 0; d < 3; ++d) {
             const float a = g.aabb[d] * (1.0f - s[d]);
@@ -303,7 +325,7 @@ __global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps,
     for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
         const uint64_t p = tile * kTile + slot;
         if (p >= M) continue;
-        float q[3];
+        float q[4];
         list_coords(g, rays, list[p], q);
         const float s = density_sum<T>(ps, q, qlane, den_w);
         if (qlane == 0) sigma[p] = activate(s, act, shift);
@@ -320,7 +342,7 @@ __global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int
     for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
         const uint64_t p = tile * kTile + slot;
         if (p >= M) continue;
-        float q[3];
+        float q[4];
         list_coords(g, rays, list[p], q);
         app_store<T>(ps, q, qlane, out + p * (uint64_t)K);
     }
@@ -393,9 +415,10 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
             if (!finish) {
                 const int s = (int)(flat - flat0);
                 const float z = lm_sample_z(g, rp, s);
-                float pt[3], q[3];
+                float pt[3], q[4];
                 lm_point(ray, z, pt);
                 lm_normalise(g, pt, q);
+                q[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q) : 0);
                 const float sig = activate(density_sum<T>(ps, q, qlane, den_w), act, shift);
                 const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
                 const float d2 = dist * distance_scale;
@@ -490,7 +513,7 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
     const uint64_t n_waves = (uint64_t)gridDim.x * kWaves;
     for (uint64_t tile_id = wave_id; tile_id < n_tiles; tile_id += n_waves) {
         // the two samples this lane gathers for (pass 0: tile row gs, pass 1: row 16 + gs)
-        float q0[3], q1[3];
+        float q0[4], q1[4];
         {
             const uint64_t p0 = tile_id * 32 + gs, p1 = p0 + 16;
             list_coords(g, rays, list[p0 < M ? p0 : M - 1], q0);
@@ -505,8 +528,9 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
 #pragma unroll
             for (int pass = 0; pass < 2; ++pass) {
                 const float *q = pass ? q1 : q0;
-                const Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-                const Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+                Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+                Taps1 t1 = line_taps(pl, pick(q, pl.axl));
+                block_taps(pl, ps.nblk, q, t2, t1);
                 float *row = tile + (pass * 16 + gs) * ROW;
 #pragma unroll
                 for (int c = V * (int)qlane; c < C; c += V * kQuad) {
@@ -607,10 +631,11 @@ int lm_check_planes(const lm_plane *planes, int32_t n, int *dtype_out, int *K_ou
     return LM_OK;
 }
 
-static PlaneSet make_set(const lm_plane *planes, int n) {
+static PlaneSet make_set(const lm_plane *planes, int n, const lm_geom *g = nullptr) {
     PlaneSet ps;
     for (int k = 0; k < LM_MAX_PLANES; ++k) ps.p[k] = planes[k < n ? k : 0];
     ps.n = n;
+    ps.nblk = g && g->div0 > 0 ? g->div0 * g->div1 : 0;
     return ps;
 }
 
@@ -667,7 +692,7 @@ extern "C" int lm_density_valid(const lm_model *m, const float *rays, const uint
     if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
     LM_REQUIRE(rays && valid_idx && counters && sigma, "null buffer");
     LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
-    const PlaneSet ps = make_set(m->density, m->n_planes);
+    const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
     const unsigned grid = (unsigned)lm_persistent_blocks(8);
     if (dtype == LM_F32)
         hipLaunchKernelGGL(k_density_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps,
@@ -692,8 +717,11 @@ extern "C" int lm_dense_alpha(const lm_model *m, const float *lin_x, const float
     if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
     LM_REQUIRE(gx > 0 && gy > 0 && gz > 0, "empty lattice %d x %d x %d", gx, gy, gz);
     LM_REQUIRE(lin_x && lin_y && lin_z && alpha, "null buffer");
+    if (g.div0 > 0)
+        LM_FAIL(LM_ERR_UNSUPPORTED, "dense alpha of a block-stacked model: the reference evaluates it per block during "
+                                    "training only");
     LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
-    const PlaneSet ps = make_set(m->density, m->n_planes);
+    const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
     const uint64_t tiles = ((uint64_t)gx * gy * gz + kTile - 1) / kTile;
     const unsigned grid = (unsigned)std::min<uint64_t>(tiles, (uint64_t)lm_persistent_blocks(8));
     if (dtype == LM_F32)
@@ -713,7 +741,7 @@ extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint3
     int dtype, K;
     if (int rc = lm_check_planes(m->app, m->n_planes, &dtype, &K)) return rc;
     LM_REQUIRE(rays && app_idx && counters && products && lm_aligned16(products), "null or misaligned buffer");
-    const PlaneSet ps = make_set(m->app, m->n_planes);
+    const PlaneSet ps = make_set(m->app, m->n_planes, &m->geom);
     const unsigned grid = (unsigned)lm_persistent_blocks(8);
     if (dtype == LM_F32)
         hipLaunchKernelGGL(k_app_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, K, rays,
@@ -750,7 +778,7 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
     LM_REQUIRE(m->mlp_packed && lm_aligned16(m->mlp_packed), "packed colour-network weights are null or misaligned");
     if (!lm_app_feat_supported(m))
         LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs a 16-bit matrix mode and equal channel counts of 16..64 in steps of 16");
-    const PlaneSet ps = make_set(m->app, m->n_planes);
+    const PlaneSet ps = make_set(m->app, m->n_planes, &m->geom);
     const int nu = m->app[0].C / 16;
     hipStream_t st = (hipStream_t)stream;
     const uint32_t *cnt = counters + LM_STAT_N_APP;
@@ -772,7 +800,7 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     int dtype;
     if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
     LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
-    const PlaneSet ps = make_set(m->density, m->n_planes);
+    const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
     const unsigned grid = (unsigned)lm_persistent_blocks(8);
     if (dtype == LM_F32)
         hipLaunchKernelGGL(k_march<float>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,

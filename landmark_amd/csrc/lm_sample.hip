@@ -215,6 +215,11 @@ int lm_check_geom(const lm_geom *g) {
         LM_REQUIRE(g->vol_dtype == LM_F32 || g->vol_dtype == LM_U8 || g->vol_dtype == LM_CELLS,
                    "occupancy volume dtype %d", g->vol_dtype);
     }
+    if (g->div0 != 0 || g->div1 != 0) {
+        LM_REQUIRE(g->div0 > 0 && g->div1 > 0 && (int64_t)g->div0 * g->div1 <= 65536, "plane division %d x %d", g->div0,
+                   g->div1);
+        LM_REQUIRE(g->blk_w > 0.0f && g->blk_h > 0.0f, "block size must be positive");
+    }
     return LM_OK;
 }
 

@@ -76,6 +76,12 @@ class GridNeRFHIP:
         self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
         self._set_alpha_mask(params.alpha_volume, params.alpha_aabb)
         # --- channel-last tables
+        self.plane_division = None if params.plane_division is None else [int(v) for v in params.plane_division]
+        self._n_blocks = 0
+        if self.plane_division is not None:
+            if params.ndims != 1:
+                raise L.LandmarkError("a block-stacked model has ndims = 1 (XY planes, z lines)")
+            self._n_blocks = self.plane_division[0] * self.plane_division[1]
         self._tables = []  # keep device tensors alive
         self._density = self._relayout_set(params.density_plane, params.density_line)
         self._app = self._relayout_set(params.app_plane, params.app_line)
@@ -147,12 +153,22 @@ class GridNeRFHIP:
         for k, (pl, ln) in enumerate(zip(planes, lines)):
             if pl.dtype not in (torch.float32, torch.float16):
                 raise L.LandmarkError(f"plane dtype {pl.dtype}")
-            P, Ln = self._relayout(pl), self._relayout(ln)
+            s = L.LmPlane()
+            if self._n_blocks:
+                # block-stacked: [1,C,B,h,w] -> [B][h][w][C], [1,C,Len,B] -> [Len][B][C]
+                if pl.dim() != 5 or pl.shape[2] != self._n_blocks or ln.shape[-1] != self._n_blocks:
+                    raise L.LandmarkError(f"plane {k}: shapes {tuple(pl.shape)}, {tuple(ln.shape)} do not hold {self._n_blocks} blocks")
+                _, Cc, B, h, w = pl.shape
+                P, Ln = self._relayout(pl.reshape(1, Cc, B * h, w)), self._relayout(ln)
+                s.H, s.W, s.C = h, w, Cc
+            else:
+                if pl.dim() != 4:
+                    raise L.LandmarkError(f"plane {k} has shape {tuple(pl.shape)}: block-stacked planes need plane_division")
+                P, Ln = self._relayout(pl), self._relayout(ln)
+                s.H, s.W, s.C = P.shape
             self._tables += [P, Ln]
             d = k // L_
-            s = L.LmPlane()
             s.plane, s.line = P.data_ptr(), Ln.data_ptr()
-            s.H, s.W, s.C = P.shape
             s.Len = Ln.shape[0]
             s.ax0, s.ax1 = MAT_MODE[d]
             s.axl = VEC_MODE[d]
@@ -236,6 +252,11 @@ class GridNeRFHIP:
             g.vol_aabb_min[:] = ab[0].tolist()
             g.vol_inv[:] = (1.0 / (ab[1] - ab[0]) * 2).tolist()
             g.vol_thre = torch.tensor(p.alpha_mask_filter_thre, dtype=torch.float32).item()
+        if self._n_blocks:
+            g.div0, g.div1 = self.plane_division
+            # the reference divides float tensors by the Python floats 2/div (gridnerf_parallel.py:304-311)
+            g.blk_w = torch.tensor(2 / g.div0, dtype=torch.float32).item()
+            g.blk_h = torch.tensor(2 / g.div1, dtype=torch.float32).item()
         self._geom_cache[S] = (g, (a_d, t_d))
         return g
 
@@ -327,6 +348,8 @@ class GridNeRFHIP:
     def getDenseAlpha(self, gridSize=None):
         """Alpha of one step at the lattice points of the AABB -> (alpha [gx,gy,gz], dense_xyz [gx,gy,gz,3])
         (gridnerf_sequential.py:321-349)."""
+        if self._n_blocks:
+            raise NotImplementedError("getDenseAlpha of a block-stacked model (per-block, training only in the reference)")
         gs = [int(v) for v in (self.gridSize if gridSize is None else gridSize)]
         lin = [torch.linspace(0, 1, g).to(self.device) for g in gs]
         samples = torch.stack(torch.meshgrid(*lin, indexing="ij"), -1)

@@ -55,6 +55,9 @@ class GridNeRFParams:
     # density through a learned projection (args.nonlinear_density, gridnerf_sequential.py:679-680, 819-822)
     nonlinear_density: bool = False
     basis_den: Optional[torch.Tensor] = None  # [1, P*L*C_d]
+    # block-stacked model ("-merged-stack" checkpoint, gridnerf_branch_parallel.py:465-527): planes are
+    # [1,C,B,h,w], lines [1,C,L,B], B = plane_division[0] * plane_division[1] blocks of the XY extent
+    plane_division: Optional[List[int]] = None
 
     # ---- derived quantities, gridnerf_sequential.py:149-164 -------------------------
     @property
@@ -116,4 +119,5 @@ class GridNeRFParams:
             embedding_app=mv(self.embedding_app),
             nonlinear_density=self.nonlinear_density,
             basis_den=mv(self.basis_den),
+            plane_division=None if self.plane_division is None else list(self.plane_division),
         )

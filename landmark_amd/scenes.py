@@ -47,6 +47,7 @@ def make_params(
     encode_app: bool = False,
     nonlinear_density: bool = False,
     n_images: int = 16,
+    plane_division: Sequence[int] = None,
     **cfg,
 ) -> GridNeRFParams:
     """Random-init model.  On `device="cpu"` the global torch RNG is seeded and used
@@ -73,8 +74,13 @@ def make_params(
             m0, m1 = MAT_MODE[i]
             v = VEC_MODE[i]
             for r in resMode:
-                planes.append(draw((1, n_comp, gridSize[m1] * r, gridSize[m0] * r)))
-                lines.append(draw((1, n_comp, gridSize[v] * r, 1)))
+                if plane_division is None:
+                    planes.append(draw((1, n_comp, gridSize[m1] * r, gridSize[m0] * r)))
+                    lines.append(draw((1, n_comp, gridSize[v] * r, 1)))
+                else:  # block-stacked layout; gridSize is the size of one block
+                    B = plane_division[0] * plane_division[1]
+                    planes.append(draw((1, n_comp, B, gridSize[m1] * r, gridSize[m0] * r)))
+                    lines.append(draw((1, n_comp, gridSize[v] * r, B)))
         return planes, lines
 
     dp, dl = one_svd(density_n_comp)
@@ -116,6 +122,7 @@ def make_params(
         embedding_app=mv(emb),
         nonlinear_density=nonlinear_density,
         basis_den=mv(basis_den),
+        plane_division=None if plane_division is None else list(plane_division),
         **cfg,
     )
 

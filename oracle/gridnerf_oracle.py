@@ -22,6 +22,9 @@ How each function is pinned (tests/test_oracle_*.py):
   mlp_render                                 fp64 numpy matmul chain
   compute_alpha / get_dense_alpha /          golden vectors (tests/golden/alphamask_*.npz) written from
   update_alpha_mask                          the reference's getDenseAlpha / updateAlphaMask
+  assign_blocks_to_samples + stacked lookup  golden vectors (tests/golden/stacked_*.npz) written from the
+                                             reference's GridNeRFBranchParallel.forward; block index and
+                                             block-relative coordinates against a plain loop
   render_chunk (composition order)           golden vectors written by
                                              tests/golden/make_golden.py from the
                                              reference's own forward
@@ -100,9 +103,36 @@ def normalize_coord(p, pts):
 # --------------------------------------------------------------------------------------
 # plane / line features
 # --------------------------------------------------------------------------------------
+def assign_blocks_to_samples(p, xyz):
+    """Normalised [M,3] -> xyzb [M,4] for a block-stacked model: x, y relative to the sample's
+    block of the plane_division grid, z unchanged, b the block index mapped to [-1,1]
+    (app/models/gridnerf_parallel.py:279-338, the path taken with ckpt_type "full")."""
+    d0, d1 = p.plane_division
+    width, height = 2 / d0, 2 / d1
+    out = torch.zeros(*xyz.shape[:-1], 4, device=xyz.device)
+    out[..., :3] = xyz
+    out[..., :2] += 1
+    out[..., 0] /= width
+    out[..., 1] /= height
+    out[..., 3] = torch.floor(out[..., 0]) * d1 + torch.floor(out[..., 1])
+    out[..., :3] = xyz
+    b = out[..., 3]
+    lo = torch.stack([-1 + (b // d1) * width, -1 + (b % d1) * height], dim=-1)
+    hi = torch.stack([-1 + (b // d1 + 1) * width, -1 + (b % d1 + 1) * height], dim=-1)
+    out[..., :2] = (out[..., :2] - lo) * 2 / (hi - lo) - 1
+    out[..., 3] = -1 + 2 * b / (d0 * d1 - 1)
+    return out
+
+
 def _coords(p, xyz):
-    """Grid-sample coordinate tensors, app/models/gridnerf_sequential.py:790-795."""
+    """Grid-sample coordinate tensors, app/models/gridnerf_sequential.py:790-795; for xyzb
+    input (block-stacked planes [1,C,B,h,w], lines [1,C,L,B]) the plane lookup is trilinear over
+    (x, y, b) and the line lookup bilinear over (b, z), app/models/gridnerf_branch_parallel.py:182-193."""
     n = p.ndims
+    if xyz.shape[-1] == 4:
+        cp = torch.stack([xyz[..., [*MAT_MODE[i], MAT_MODE[i][1] + 2]] for i in range(n)]).view(n, 1, -1, 1, 3)
+        cl = torch.stack([xyz[..., [VEC_MODE[i] + 1, VEC_MODE[i]]] for i in range(n)]).view(n, -1, 1, 2)
+        return cp, cl
     cp = torch.stack([xyz[..., MAT_MODE[i]] for i in range(n)]).view(n, -1, 1, 2)
     cl = torch.stack([xyz[..., VEC_MODE[i]] for i in range(n)])
     cl = torch.stack((torch.zeros_like(cl), cl), dim=-1).view(n, -1, 1, 2)
@@ -274,6 +304,12 @@ def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False, a
     rgb = torch.zeros((*xyz.shape[:2], 3), device=xyz.device)
     if ray_valid.any():
         xyz = normalize_coord(p, xyz)
+        if getattr(p, "plane_division", None):
+            # gridnerf_parallel.py:765-771, 918-924: valid samples get block-relative coordinates
+            xyzb = torch.zeros(*xyz.shape[:-1], 4, device=xyz.device)
+            xyzb[..., :3] = xyz
+            xyzb.masked_scatter_(ray_valid.unsqueeze(-1).expand(-1, -1, 4), assign_blocks_to_samples(p, xyz[ray_valid]))
+            xyz = xyzb
         sigma[ray_valid] = feature2density(p, density_feature(p, xyz[ray_valid]))
 
     _, weight, _ = raw2alpha(sigma, dists * p.distance_scale)

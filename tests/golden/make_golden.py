@@ -278,7 +278,105 @@ def main_alpha():
               f"{arrays['new_volume'].size} new_aabb {arrays['new_aabb'].tolist()} -> {os.path.getsize(path)/1024:.0f} KB")
 
 
+STACKED_CASES = [
+    # block-stacked ("-merged-stack") models rendered on one device: planes [1,C,B,h,w], lines [1,C,L,B]
+    dict(name="hull_softplus_div2x3", grid=[5, 4, 6], div=[2, 3], act="softplus", shift=0.0, res=[1], opt=1, mask=True, thre=0.0, S=16, boost=8.0),
+    dict(name="aabb_relu_L2_div3x2", grid=[4, 5, 5], div=[3, 2], act="relu", shift=-10.0, res=[1, 2], opt=0, mask=False, thre=0.0, S=20, boost=14.0, sr=0.25),
+    dict(name="hull_relu_div2x2_encodeapp", grid=[4, 4, 5], div=[2, 2], act="relu", shift=-10.0, res=[1], opt=1, mask=True, thre=0.5, S=16, boost=12.0, encode_app=True, app_code=2),
+]
+
+
+def main_stacked():
+    """Fixtures stacked_*.npz from GridNeRFBranchParallel.forward with ckpt_type "full"."""
+    import tempfile
+
+    _install_stand_ins()
+    sys.path.insert(0, REF)
+    from app.models.alpha_mask import AlphaGridMask  # noqa: E402
+    from app.models.gridnerf_branch_parallel import GridNeRFBranchParallel  # noqa: E402
+
+    for ci, c in enumerate(STACKED_CASES):
+        torch.manual_seed(500 + ci)
+        aabb = torch.tensor([[-1.0, -1.2, -0.8], [1.1, 1.0, 0.9]])
+        B = c["div"][0] * c["div"][1]
+        gw, gh, gl = c["grid"]
+        sd = {}
+        for k, r in enumerate(c["res"]):
+            sd[f"density_plane.{k}"] = 0.1 * c["boost"] * torch.randn(1, 16, B, gh * r, gw * r)
+            sd[f"density_line.{k}"] = 0.1 * torch.randn(1, 16, gl * r, B)
+            sd[f"app_plane.{k}"] = 0.1 * torch.randn(1, 48, B, gh * r, gw * r)
+            sd[f"app_line.{k}"] = 0.1 * torch.randn(1, 48, gl * r, B)
+        with tempfile.TemporaryDirectory() as tmp:
+            path = os.path.join(tmp, "x-merged-stack.th")
+            torch.save({"kwargs": {}, "state_dict": sd}, path)
+            args = _args(
+                ndims=1, resMode=c["res"], sampling_opt=c["opt"], n_importance=max(c["S"], 8), alpha_mask_filter_thre=c["thre"],
+                encode_app=bool(c.get("encode_app")), ckpt=path, ckpt_type="full", plane_division=c["div"], branch_parallel=True,
+                plane_parallel=False, channel_parallel=False, DDP=False, local_rank=0, part=0, model_parallel_degree=B,
+            )
+            model = GridNeRFBranchParallel(
+                aabb, c["grid"], "cpu",
+                density_n_comp=[16] * 3, appearance_n_comp=[48] * 3, app_dim=27,
+                near_far=[0.4, 4.0], density_shift=c["shift"], distance_scale=25, rayMarch_weight_thres=0.001,
+                pos_pe=2, view_pe=2, fea_pe=2, featureC=128, step_ratio=c.get("sr", 2.0),
+                fea2denseAct=c["act"], args=args, is_train=False,
+            )
+            model.load({"state_dict": dict(sd)})
+        model.eval()
+        app_code = torch.tensor(0)
+        if c.get("encode_app"):
+            model.embedding_app = torch.nn.Embedding(8, 48)
+            app_code = torch.tensor(c["app_code"])
+        with torch.no_grad():
+            if c["mask"]:
+                g = torch.Generator().manual_seed(60 + ci)
+                vol = (torch.rand(5, 7, 6, generator=g) < 0.7).float()
+                mask_aabb = aabb + torch.tensor([[0.05, -0.02, 0.0], [0.0, 0.03, -0.04]])
+                model.alphaMask = AlphaGridMask("cpu", mask_aabb, vol)
+            rays = _camera_rays(7, (1.4, -1.1, 1.9), 21 + ci) if c["opt"] else _generic_rays(40, 21 + ci)
+            out = model(rays, app_code=app_code, is_train=False, white_bg=True, N_samples=c["S"])
+            out_black = model(rays, app_code=app_code, is_train=False, white_bg=False, N_samples=c["S"])
+            if isinstance(out, tuple):
+                out, out_black = out[0], out_black[0]
+            # sub-function vectors: block assignment and the stacked lookups on every in-box sample
+            if c["opt"]:
+                pts, _, z, inside = model.sample_ray_within_hull(rays[:, :3], rays[:, 3:6], is_train=False, N_samples=model.n_importance)
+            else:
+                pts, _, z, inside = model.sample_ray(rays[:, :3], rays[:, 3:6], is_train=False, N_samples=c["S"])
+            q = model.normalize_coord(pts)
+            _, xyzb = model.assign_blocks_to_samples(q, inside, is_train=False)
+            dens = model.compute_densityfeature(xyzb, use_xyzb=True)
+            appf = model.compute_appfeature(xyzb, use_xyzb=True)
+            store = {
+                "rays": rays, "rgb_map": out["rgb_map"], "depth_map": out["depth_map"], "rgb_map_black": out_black["rgb_map"],
+                "sub_z": z, "sub_inside": inside, "sub_xyz": q[inside], "sub_xyzb": xyzb, "sub_density_feature": dens,
+                "sub_app_feature": appf, "aabb": aabb,
+            }
+            if c["mask"]:
+                store["alpha_volume"], store["alpha_aabb"] = vol, mask_aabb
+            for k, v in model.state_dict().items():
+                store["sd." + k] = v
+        cfg = dict(
+            grid=c["grid"], ndims=1, resMode=c["res"], sampling_opt=c["opt"], N_samples=c["S"], n_importance=int(model.n_importance),
+            near_far=[0.4, 4.0], density_shift=c["shift"], fea2denseAct=c["act"], step_ratio=float(model.step_ratio),
+            thre=c["thre"], nSamples=int(model.nSamples), stepSize=float(model.stepSize), encode_app=bool(c.get("encode_app")),
+            nonlinear_density=False, app_code=c.get("app_code"), plane_division=c["div"],
+        )
+        arrays = {k: (v.detach().cpu().numpy() if torch.is_tensor(v) else np.asarray(v)) for k, v in store.items()}
+        arrays["cfg_json"] = np.frombuffer(__import__("json").dumps(cfg).encode(), dtype=np.uint8)
+        path = os.path.join(HERE, f"stacked_{c['name']}.npz")
+        np.savez_compressed(path, **arrays)
+        blocks = sorted(set(((xyzb[:, 3] + 1) / 2 * (B - 1)).round().long().tolist()))
+        print(f"stacked_{c['name']}: rays {tuple(rays.shape)} in-box {int(inside.sum())} blocks hit {blocks} "
+              f"rgb mean {out['rgb_map'].mean():.4f} min {out['rgb_map'].min():.3f} -> {os.path.getsize(path)/1024:.0f} KB")
+
+
 if __name__ == "__main__":
-    if "--alpha-only" not in sys.argv:
+    only = [a for a in sys.argv[1:] if a.startswith("--only=")]
+    which = only[0][len("--only=") :].split(",") if only else ["forward", "alpha", "stacked"]
+    if "forward" in which:
         main()
-    main_alpha()
+    if "alpha" in which:
+        main_alpha()
+    if "stacked" in which:
+        main_stacked()

@@ -19,6 +19,10 @@ def alphamask_names():
     return sorted(os.path.basename(p)[len("alphamask_") : -len(".npz")] for p in glob.glob(os.path.join(GOLDEN_DIR, "alphamask_*.npz")))
 
 
+def stacked_names():
+    return sorted(os.path.basename(p)[len("stacked_") : -len(".npz")] for p in glob.glob(os.path.join(GOLDEN_DIR, "stacked_*.npz")))
+
+
 def load_golden(name, kind="forward"):
     """(params, data dict of tensors, cfg) for one fixture written by golden/make_golden.py."""
     z = np.load(os.path.join(GOLDEN_DIR, f"{kind}_{name}.npz"))
@@ -55,5 +59,6 @@ def load_golden(name, kind="forward"):
         embedding_app=sd.get("embedding_app.weight"),
         nonlinear_density=cfg.get("nonlinear_density", False),
         basis_den=sd.get("basis_den.weight"),
+        plane_division=cfg.get("plane_division"),
     )
     return p, data, cfg

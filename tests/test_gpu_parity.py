@@ -12,7 +12,7 @@ import torch
 
 from landmark_amd import scenes
 from oracle import gridnerf_oracle as O
-from tests.helpers import alphamask_names, golden_names, load_golden
+from tests.helpers import alphamask_names, golden_names, load_golden, stacked_names
 
 pytestmark = pytest.mark.gpu
 
@@ -411,3 +411,50 @@ def test_mask_update_random_scene_then_render(gpu_lib, act, shift, res, with_mas
     assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
     res_, _ = m(rays)
     assert (res_["rgb_map"].cpu() - ref["rgb_map"]).abs().max().item() <= RGB_TOL_F32
+
+
+# ------------------------------------------------------------------------------------ block-stacked models
+@pytest.mark.parametrize("name", stacked_names())
+def test_stacked_model_golden(gpu_lib, name):
+    p, d, cfg = load_golden(name, kind="stacked")
+    code = cfg.get("app_code")
+    m = _model(p)
+    ref = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], app_code=code, return_aux=True)
+    cull = m.sample_cull(d["rays"], N_samples=cfg["N_samples"])
+    assert torch.equal(cull["ray_valid"].cpu(), ref["ray_valid"])
+    # densities of the valid samples through the stage entry point
+    sigma = m.density_valid(cull)
+    assert (sigma.cpu() - ref["sigma"][ref["ray_valid"]]).abs().max().item() <= 1e-5 * max(1.0, ref["sigma"].max().item())
+    for white, key in ((True, "rgb_map"), (False, "rgb_map_black")):
+        out, _ = m(d["rays"], app_code=code, white_bg=white, N_samples=cfg["N_samples"])
+        assert (out["rgb_map"].cpu() - d[key]).abs().max().item() <= RGB_TOL_F32
+        assert (out["depth_map"].cpu() - d["depth_map"]).abs().max().item() <= RGB_TOL_F32
+
+
+@pytest.mark.parametrize("div,res,prec", [((2, 3), (1,), "f32"), ((4, 2), (1, 2), "f16x2"), ((3, 3), (1, 2, 4), "f16x2")])
+def test_stacked_model_random_scene(gpu_lib, div, res, prec):
+    p = scenes.make_params(seed=11, gridSize=(10, 9, 12), near_far=[0.5, 4.5], n_importance=96, sampling_opt=1,
+                           density_shift=0.0, resMode=res, ndims=1, plane_division=div)
+    for t in p.density_plane:
+        t.mul_(8.0)
+    rays = scenes.pinhole_rays(72, 72, 60.0, scenes.sphere_pose(2.5, 7))
+    ref = O.render_chunk(p, rays, return_aux=True)
+    assert ref["app_mask"].any()
+    out, _ = _model(p, mlp_precision=prec)(rays)
+    band = ((ref["weight"] - p.rayMarch_weight_thres).abs() < 2e-7).any(-1)
+    assert (out["rgb_map"].cpu() - ref["rgb_map"])[~band].abs().max().item() <= RGB_TOL_F32
+    assert (out["depth_map"].cpu() - ref["depth_map"])[~band].abs().max().item() <= RGB_TOL_F32
+    assert int(band.sum()) <= max(2, rays.shape[0] // 500)
+
+
+def test_stacked_checkpoint_round_trip(gpu_lib, tmp_path):
+    from landmark_amd import checkpoint
+
+    p, d, cfg = load_golden(stacked_names()[0], kind="stacked")
+    path = str(tmp_path / "x-merged-stack.th")
+    checkpoint.save_checkpoint(p, path)
+    q = checkpoint.load_checkpoint(path, resMode=cfg["resMode"], ndims=1, sampling_opt=cfg["sampling_opt"],
+                                   n_importance=cfg["n_importance"], alpha_mask_filter_thre=cfg["thre"])
+    assert q.plane_division == cfg["plane_division"] and q.density_plane[0].dim() == 5
+    out, _ = _model(q)(d["rays"], N_samples=cfg["N_samples"])
+    assert (out["rgb_map"].cpu() - d["rgb_map"]).abs().max().item() <= RGB_TOL_F32

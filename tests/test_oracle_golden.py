@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import gridnerf_oracle as O
-from tests.helpers import alphamask_names, golden_names, load_golden
+from tests.helpers import alphamask_names, golden_names, load_golden, stacked_names
 
 NAMES = golden_names()
 
@@ -107,3 +107,34 @@ def test_alpha_mask_pool_brute_force():
                         lo[k] = v if lo[k] is None else min(lo[k], v)
                         hi[k] = v if hi[k] is None else max(hi[k], v)
     assert new_aabb[0].tolist() == lo and new_aabb[1].tolist() == hi
+
+
+@pytest.mark.parametrize("name", stacked_names())
+def test_stacked_model_matches_reference(name):
+    """Block-stacked planes rendered on one device (tests/golden/stacked_*.npz, written from
+    GridNeRFBranchParallel.forward with ckpt_type "full")."""
+    p, d, cfg = load_golden(name, kind="stacked")
+    code = cfg.get("app_code")
+    out = O.render_chunk(p, d["rays"], white_bg=True, N_samples=cfg["N_samples"], app_code=code, return_aux=True)
+    assert torch.equal(out["rgb_map"], d["rgb_map"]) and torch.equal(out["depth_map"], d["depth_map"])
+    out_b = O.render_chunk(p, d["rays"], white_bg=False, N_samples=cfg["N_samples"], app_code=code)
+    assert torch.equal(out_b["rgb_map"], d["rgb_map_black"])
+    assert out["app_mask"].any()
+    xyzb = O.assign_blocks_to_samples(p, d["sub_xyz"])
+    assert torch.equal(xyzb, d["sub_xyzb"])
+    assert torch.equal(O.density_feature(p, xyzb), d["sub_density_feature"])
+    assert torch.equal(O.app_feature(p, xyzb), d["sub_app_feature"])
+
+
+def test_block_assignment_plain_loop():
+    """Block index and block-relative coordinates against scalar arithmetic in float64."""
+    p, d, cfg = load_golden(stacked_names()[0], kind="stacked")
+    d0, d1 = cfg["plane_division"]
+    g = torch.Generator().manual_seed(3)
+    xyz = torch.rand(500, 3, generator=g) * 1.98 - 0.99
+    out = O.assign_blocks_to_samples(p, xyz)
+    for (x, y, z), (lx, ly, lz, b) in zip(xyz.double().tolist(), out.double().tolist()):
+        bx, by = int((x + 1) / (2 / d0)), int((y + 1) / (2 / d1))
+        assert round((b + 1) / 2 * (d0 * d1 - 1)) == bx * d1 + by
+        assert lz == z
+        assert abs(lx - (((x + 1) - bx * 2 / d0) * d0 - 1)) < 1e-5 and abs(ly - (((y + 1) - by * 2 / d1) * d1 - 1)) < 1e-5
