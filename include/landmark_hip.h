@@ -184,7 +184,8 @@ int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, int32_t gz, f
  *   rays        [N,6]  origin, direction
  *   bitmap      [ceil(N*S/64)] uint64, bit (i & 63) of word i>>6 = sample i is valid
  *   word_prefix [ceil(N*S/64)] uint32, number of valid samples before each word
- *   valid_idx   [N*S] uint32 capacity, ascending flat indices of valid samples
+ *   valid_idx   [N*S] uint32 capacity, ascending flat indices of valid samples; may be NULL
+ *               (not written) when the caller walks the bitmap instead
  *   counters    [LM_STAT_WORDS] uint32, counters[LM_STAT_N_VALID] = number of valid samples
  *   z_out       optional [N*S] sample depths (NULL to skip)
  *   scratch     lm_sample_cull_scratch_bytes(N,S) bytes

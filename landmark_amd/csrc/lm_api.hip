@@ -97,8 +97,6 @@ struct Workspace {
     uint64_t *bitmap;
     uint32_t *word_prefix;
     void *cull_scratch;
-    uint32_t *valid_idx;
-    float *sigma;
     float *w_valid;
     uint32_t *app_first;
     uint32_t *app_cnt;
@@ -128,8 +126,6 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products)
     w.bitmap = (uint64_t *)take(n_words * 8);
     w.word_prefix = (uint32_t *)take(n_words * 4);
     w.cull_scratch = take(lm_sample_cull_scratch_bytes(N, S));
-    w.valid_idx = (uint32_t *)take(total * 4);
-    w.sigma = (float *)take(total * 4);
     w.w_valid = (float *)take(total * 4);
     w.app_first = (uint32_t *)take((uint64_t)N * 4);
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
@@ -189,7 +185,7 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     };
     mark(0);
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
-    if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, w.valid_idx, cnt, nullptr, w.cull_scratch, st))
+    if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, nullptr, cnt, nullptr, w.cull_scratch, st))
         return rc;
     if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.ray_list, cnt + LM_STAT_N_ACTIVE, w.acc, depth_map,
                                        w.app_cnt, w.p_end, st))

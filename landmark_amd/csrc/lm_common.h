@@ -190,6 +190,37 @@ __device__ __forceinline__ float lm_alpha_lookup(const lm_geom &g, const float *
     return out;
 }
 
+// lm_alpha_lookup(g, pt) > 0 for a cell table, without forming the sum: every term is a
+// product of three weights in [0, 1] (never small enough to underflow: a weight is a difference
+// of numbers below 2^24 with spacing >= 2^-24 of their size), so the sum is positive exactly when a
+// set corner has three non-zero weights.  The lower weight (f + 1) - i is never zero; the upper
+// weight i - f is zero when the coordinate is an integer.
+__device__ __forceinline__ bool lm_cells_positive(const lm_geom &g, const float *pt) {
+    float c[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        float d = pt[k] - g.vol_aabb_min[k];
+        float m = d * g.vol_inv[k];
+        c[k] = m - 1.0f;
+    }
+    const int W = g.vw, H = g.vh, D = g.vd;
+    const float ix = ((c[0] + 1.0f) / 2.0f) * (float)(W - 1);
+    const float iy = ((c[1] + 1.0f) / 2.0f) * (float)(H - 1);
+    const float iz = ((c[2] + 1.0f) / 2.0f) * (float)(D - 1);
+    float fx = floorf(ix), fy = floorf(iy), fz = floorf(iz);
+    unsigned live = 0xFFu;
+    if (ix - fx == 0.0f) live &= 0x55u;  // corners with xx = 1 weigh nothing
+    if (iy - fy == 0.0f) live &= 0x33u;
+    if (iz - fz == 0.0f) live &= 0x0Fu;
+    fx = fminf(fmaxf(fx, -2.0f), (float)W);
+    fy = fminf(fmaxf(fy, -2.0f), (float)H);
+    fz = fminf(fmaxf(fz, -2.0f), (float)D);
+    const int x0 = (int)fx, y0 = (int)fy, z0 = (int)fz;
+    if (x0 < -1 || x0 >= W || y0 < -1 || y0 >= H || z0 < -1 || z0 >= D) return false;
+    const size_t ci = ((size_t)(z0 + 1) * (H + 1) + (y0 + 1)) * (W + 1) + (x0 + 1);
+    return (reinterpret_cast<const uint8_t *>(g.vol)[ci] & live) != 0u;
+}
+
 // Sample validity = inside the AABB and (no volume or lookup > threshold)
 __device__ __forceinline__ bool lm_sample_valid(const lm_geom &g, const float *pt) {
     bool ok = lm_inside(g, pt);

@@ -66,6 +66,53 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *
     }
 }
 
+// Same decisions, one lane per (ray, bitmap word), for S = 64 * WPR with WPR in {1, 2, 4}.  A
+// lane walks the 64 samples of its word and keeps the bits in a register; the 64 lanes of a
+// wave are 64 neighbouring rays at the same depth, so their occupancy lookups fall into the
+// same few cache lines (a wave of 64 samples along one ray touches 64 different ones), and the
+// per-ray work (slab test or hull distance) is done once per word instead of once per sample.
+// A workgroup covers 256 consecutive words = 4 of the 64-word groups k_scan_blocks counts.
+template <int WPR>
+__global__ __launch_bounds__(kBlock) void k_sample_cull_rays(lm_geom g, const float *__restrict__ rays, uint32_t N,
+                                                             uint64_t nb, uint64_t *__restrict__ bitmap,
+                                                             uint32_t *__restrict__ block_count) {
+    __shared__ uint32_t s_cnt[4];
+    const unsigned lane = lm_lane(), wave = threadIdx.x / LM_WAVE;
+    if (threadIdx.x < 4) s_cnt[threadIdx.x] = 0;
+    __syncthreads();
+    constexpr unsigned kRays = kBlock / WPR;  // rays per workgroup
+    const unsigned j = wave % WPR;
+    const unsigned ray_local = (wave / WPR) * 64 + lane;
+    const uint64_t r = (uint64_t)blockIdx.x * kRays + ray_local;
+    uint64_t bits = 0;
+    if (r < N) {
+        float ray[6];
+        const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
+        const float2 a = rp2[0], b = rp2[1], c = rp2[2];
+        ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+        const float rp = lm_ray_param(g, ray);
+        const bool cells0 = g.vol && g.vol_dtype == LM_CELLS && g.vol_thre == 0.0f;
+#pragma unroll 4
+        for (int i = 0; i < 64; ++i) {
+            const float z = lm_sample_z(g, rp, (int)j * 64 + i);
+            float pt[3];
+            lm_point(ray, z, pt);
+            bool ok;
+            if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
+            else ok = lm_sample_valid(g, pt);
+            bits |= (uint64_t)ok << i;
+        }
+        bitmap[r * WPR + j] = bits;
+    }
+    const uint32_t cnt = (uint32_t)__popcll(bits);
+    if (cnt) atomicAdd(&s_cnt[(ray_local * WPR + j) / 64], cnt);
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        const uint64_t bi = (uint64_t)blockIdx.x * 4 + threadIdx.x;
+        if (bi < nb) block_count[bi] = s_cnt[threadIdx.x];
+    }
+}
+
 // exclusive scan of n counts by one workgroup of 1024 threads; total -> *total_out
 __global__ __launch_bounds__(1024) void k_scan_blocks(const uint32_t *__restrict__ in, uint32_t *__restrict__ out,
                                                       uint32_t n, uint32_t *__restrict__ total_out) {
@@ -120,7 +167,7 @@ __global__ __launch_bounds__(kBlock) void k_emit(const uint64_t *__restrict__ bi
         const uint64_t w = wb + wi;
         if (w >= n_words) break;
         const uint64_t bits = bitmap[w];
-        if ((bits >> lane) & 1ull) valid_idx[s_pref[wi] + lm_mbcnt(bits)] = (uint32_t)(w * 64 + lane);
+        if (valid_idx && ((bits >> lane) & 1ull)) valid_idx[s_pref[wi] + lm_mbcnt(bits)] = (uint32_t)(w * 64 + lane);
     }
 }
 
@@ -240,16 +287,29 @@ extern "C" int lm_sample_cull(const lm_geom *geom, const float *rays, int64_t N,
         LM_CHECK_LAUNCH("k_scan_blocks");
         return LM_OK;
     }
-    LM_REQUIRE(rays && bitmap && word_prefix && valid_idx && scratch, "null buffer");
+    LM_REQUIRE(rays && bitmap && word_prefix && scratch, "null buffer");
     LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
     LM_REQUIRE(lm_aligned16(bitmap) && lm_aligned16(scratch), "bitmap and scratch must be 16-byte aligned");
     const uint64_t n_words = (total + 63) / 64;
     const uint64_t nb = n_blocks_for(n_words);
     uint32_t *block_count = (uint32_t *)scratch;
     uint32_t *block_off = block_count + nb;
-    hipLaunchKernelGGL(k_sample_cull, dim3((unsigned)nb), dim3(kBlock), 0, st, *geom, rays, total, n_words, bitmap,
-                       block_count, z_out);
-    LM_CHECK_LAUNCH("k_sample_cull");
+    const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
+    if (!z_out && (wpr == 1 || wpr == 2 || wpr == 4)) {
+        const unsigned groups = (unsigned)((n_words + 255) / 256);
+#define LM_CULL_RAYS(W_)                                                                                              \
+    hipLaunchKernelGGL(k_sample_cull_rays<W_>, dim3(groups), dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, nb, bitmap, \
+                       block_count)
+        if (wpr == 1) LM_CULL_RAYS(1);
+        else if (wpr == 2) LM_CULL_RAYS(2);
+        else LM_CULL_RAYS(4);
+#undef LM_CULL_RAYS
+        LM_CHECK_LAUNCH("k_sample_cull_rays");
+    } else {
+        hipLaunchKernelGGL(k_sample_cull, dim3((unsigned)nb), dim3(kBlock), 0, st, *geom, rays, total, n_words, bitmap,
+                           block_count, z_out);
+        LM_CHECK_LAUNCH("k_sample_cull");
+    }
     hipLaunchKernelGGL(k_scan_blocks, dim3(1), dim3(1024), 0, st, (const uint32_t *)block_count, block_off,
                        (uint32_t)nb, counters + LM_STAT_N_VALID);
     LM_CHECK_LAUNCH("k_scan_blocks");

@@ -62,6 +62,46 @@ def test_sample_cull_random_scene_bit_exact(gpu_lib, opt, S, thre):
     assert torch.equal(out["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
 
 
+@pytest.mark.parametrize("opt,S,thre,mask,occ", [
+    (1, 64, 0.0, True, "auto"), (1, 128, 0.0, True, "auto"), (1, 256, 0.0, True, "auto"), (1, 128, 0.5, True, "auto"),
+    (1, 128, 0.0, True, "f32"), (1, 128, 0.0, False, "auto"), (0, 64, 0.0, True, "auto"), (0, 128, 0.98, True, "u8"),
+])
+def test_sample_cull_ray_per_lane_kernel(gpu_lib, opt, S, thre, mask, occ):
+    """S = 64, 128, 256 without depths takes the kernel with one lane per (ray, bitmap word): same masks, same
+    list, same counts as the oracle and as the sample-per-lane kernel (taken when depths are asked for)."""
+    p = _scene(opt=opt, S=S, thre=thre, with_mask=mask, step_ratio=0.4)
+    rays = scenes.pinhole_rays(101, 77, 80.0, scenes.sphere_pose(2.5, 5))  # 7777 rays: ragged last workgroup
+    ref = O.render_chunk(p, rays, N_samples=S, return_aux=True)
+    m = _model(p, occupancy=occ)
+    a = m.sample_cull(rays, N_samples=S, want_z=False)
+    b = m.sample_cull(rays, N_samples=S, want_z=True)
+    assert 0 < int(ref["ray_valid"].sum()) < ref["ray_valid"].numel()
+    assert torch.equal(a["ray_valid"].cpu(), ref["ray_valid"])
+    assert torch.equal(a["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
+    assert a["n_valid"] == b["n_valid"] and torch.equal(a["bitmap"], b["bitmap"]) and torch.equal(a["word_prefix"], b["word_prefix"])
+
+
+def test_occupancy_lookup_on_voxel_centres(gpu_lib):
+    """Sample points that fall exactly on voxel centres and faces of the occupancy grid (zero upper weights):
+    the positive-lookup shortcut must agree with the summed lookup."""
+    p = _scene(with_mask=False, S=64, opt=0, step_ratio=1.0, grid=(9, 9, 9))
+    p.aabb = torch.tensor([[-1.0, -1.0, -1.0], [1.0, 1.0, 1.0]])
+    g = torch.Generator().manual_seed(5)
+    p.alpha_volume = (torch.rand(9, 9, 9, generator=g) < 0.3).float()
+    p.alpha_aabb = p.aabb.clone()
+    # axis-parallel rays through lattice lines: x, y on voxel centres, z stepping by exactly one voxel (0.25)
+    xs = torch.linspace(-1, 1, 9)
+    o = torch.stack(torch.meshgrid(xs, xs, indexing="ij"), -1).reshape(-1, 2)
+    rays = torch.cat([o, torch.full((81, 1), -1.5), torch.zeros(81, 2), torch.ones(81, 1)], 1)
+    p.near_far = [0.5, 4.0]
+    S = 64
+    ref = O.render_chunk(p, rays, N_samples=S, return_aux=True)
+    assert 0 < int(ref["ray_valid"].sum())
+    for occ in ("auto", "f32"):
+        out = _model(p, occupancy=occ).sample_cull(rays, N_samples=S, want_z=False)
+        assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
+
+
 @pytest.mark.parametrize("occupancy", ["f32", "u8", "cells"])
 def test_occupancy_storages_agree_bit_for_bit(gpu_lib, occupancy):
     p = _scene(S=128, thre=0.5)
