@@ -132,8 +132,11 @@ def bench_frame(args, workload):
                                    GBps=round(n_marched * dens_B / (stage_ms[1] * 1e-3) / 1e9, 1))
     stages["app_gather"].update(bytes_per_sample=app_B, GBps=round(n_app * app_B / max(stage_ms[3], 1e-9) / 1e6, 1))
     stages["colour"].update(TFLOPs=round(n_app * (MLP_FLOP_PER_ROW + 2 * model.K_app * 27) / max(stage_ms[4], 1e-9) / 1e9, 2))
-    cull_B = 32 + 0.125  # 8 corner loads of the float volume per in-box sample (upper bound: every sample), bitmap out
-    stages["cull"].update(GBps=round((N * S * cull_B + n_valid * 4) / (stage_ms[0] * 1e-3) / 1e9, 1))
+    # occupancy lookups: 1 byte per sample from the cell table (8 x 4 bytes with a float volume), upper bound
+    # every sample; 1 bit per sample and 24 bytes per ray besides
+    cull_B = (1 if model._vol_dtype == L.LM_CELLS else 32 if model._vol is not None else 0) + 0.125
+    stages["cull"].update(bytes_per_sample=cull_B, Gsamples_per_s=round(N * S / (stage_ms[0] * 1e-3) / 1e9, 1),
+                          GBps=round((N * S * cull_B + N * 24) / (stage_ms[0] * 1e-3) / 1e9, 1))
     stages["app_list"].update(GBps=round((n_marched * 4 + N * S / 8 + n_app * 8 + N * 16) / (stage_ms[2] * 1e-3) / 1e9, 1))
 
     # dominant kernel -> roofline object

@@ -80,13 +80,16 @@ int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float
 int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
                         const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream);
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
-int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *ray_list,
-                          uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt, uint32_t *p_end,
-                          hipStream_t stream);
-int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, const float *w_valid,
+int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
+                          uint32_t *ray_list, uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt,
+                          uint32_t *p_end, hipStream_t stream);
+int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
+                         uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
+                         uint32_t *app_cnt, uint32_t *p_end, hipStream_t st);
+int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
                         float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
                         uint32_t *app_idx, float *app_w, uint32_t *app_count, hipStream_t stream);
-int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *word_prefix,
+int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
                     const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st);
 int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
@@ -100,6 +103,7 @@ struct Workspace {
     float *w_valid;
     uint32_t *app_first;
     uint32_t *app_cnt;
+    uint32_t *p_first;
     uint32_t *p_end;
     uint32_t *ray_list;
     uint32_t *app_idx;
@@ -129,6 +133,7 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products)
     w.w_valid = (float *)take(total * 4);
     w.app_first = (uint32_t *)take((uint64_t)N * 4);
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
+    w.p_first = (uint32_t *)take((uint64_t)N * 4);
     w.p_end = (uint32_t *)take((uint64_t)N * 4);
     w.ray_list = (uint32_t *)take((uint64_t)N * 4);
     w.app_idx = (uint32_t *)take(cap * 4);
@@ -185,17 +190,24 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     };
     mark(0);
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
-    if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, nullptr, cnt, nullptr, w.cull_scratch, st))
-        return rc;
-    if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.ray_list, cnt + LM_STAT_N_ACTIVE, w.acc, depth_map,
-                                       w.app_cnt, w.p_end, st))
-        return rc;
+    // sample counts of 64, 128 or 256: one launch decides the samples and sets the rays up; otherwise the
+    // stage-level cull (scan + per-word prefix) followed by the list kernel
+    int rc_setup = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE,
+                                        cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, st);
+    if (rc_setup < 0) return rc_setup;
+    if (rc_setup > 0) {
+        if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, nullptr, cnt, nullptr, w.cull_scratch, st))
+            return rc;
+        if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE,
+                                           w.acc, depth_map, w.app_cnt, w.p_end, st))
+            return rc;
+    }
     mark(LM_STAGE_CULL);
-    if (int rc = lm_launch_march(m, rays, w.bitmap, w.word_prefix, w.ray_list, cnt + LM_STAT_N_ACTIVE, cnt + LM_STAT_QUEUE,
+    if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE, cnt + LM_STAT_QUEUE,
                                  w.w_valid, w.acc, depth_map, w.app_cnt, w.p_end, cnt + LM_STAT_N_MARCHED, st))
         return rc;
     mark(LM_STAGE_DENSITY);
-    if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.word_prefix, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
+    if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.p_first, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
                                      w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, st))
         return rc;
     mark(LM_STAGE_WEIGHTS);

@@ -251,6 +251,15 @@ struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
         pos = pf[w] + (uint32_t)__popcll(raw & below);
         bits = mask_tail(raw & ~below);
     }
+    // same walk when the compact position of the first sample is known (a per-ray table)
+    __device__ __forceinline__ void start_at(const uint64_t *bm, uint64_t flat0, uint64_t flat1_, uint32_t pos0) {
+        bitmap = bm; prefix = nullptr; flat1 = flat1_;
+        w = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
+        const unsigned b0 = (unsigned)(flat0 & 63);
+        const uint64_t below = b0 ? ((1ull << b0) - 1ull) : 0ull;
+        pos = pos0;
+        bits = mask_tail(bm[w] & ~below);
+    }
     __device__ __forceinline__ uint64_t mask_tail(uint64_t x) const {
         if (w == w_last) {
             const unsigned e = (unsigned)(flat1 & 63);

@@ -126,9 +126,10 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
 }
 
 // Rays that have at least one valid sample, for the marching kernel's queue; the others get
-// their (zero) results here.
+// their (zero) results here.  p_first[r] = compact position of the ray's first valid sample.
 __global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
                                                         const uint32_t *__restrict__ word_prefix,
+                                                        uint32_t *__restrict__ p_first,
                                                         uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
                                                         float *__restrict__ acc, float *__restrict__ depth,
                                                         uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end) {
@@ -138,6 +139,7 @@ __global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const
     if (r < N) {
         BitWalk it;
         it.start(bitmap, word_prefix, r * (uint64_t)S, (r + 1) * (uint64_t)S);
+        p_first[r] = it.pos;
         uint64_t flat;
         any = it.next(flat);
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = it.pos; }
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const
 // Appearance list from stored weights: a contiguous slot range per ray (wave prefix + one
 // atomic), filled in sample order from the weights of the ray's samples [first, p_end).
 __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
-                                                      const uint32_t *__restrict__ word_prefix,
+                                                      const uint32_t *__restrict__ p_first,
                                                       const float *__restrict__ w_valid, float weight_thres,
                                                       const uint32_t *__restrict__ app_cnt,
                                                       const uint32_t *__restrict__ p_end,
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const u
     app_first[r] = slot;
     if (cnt) {
         BitWalk it;
-        it.start(bitmap, word_prefix, r * (uint64_t)S, (r + 1) * (uint64_t)S);
+        it.start_at(bitmap, r * (uint64_t)S, (r + 1) * (uint64_t)S, p_first[r]);
         const uint32_t end = p_end[r];
         uint64_t flat;
         for (uint32_t p = it.pos; p < end; ++p) {
@@ -237,21 +239,21 @@ int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
     return LM_OK;
 }
 
-int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *ray_list,
-                          uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt, uint32_t *p_end,
-                          hipStream_t stream) {
+int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
+                          uint32_t *ray_list, uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt,
+                          uint32_t *p_end, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(k_active_rays, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, ray_list,
-                       n_active, acc, depth, app_cnt, p_end);
+    hipLaunchKernelGGL(k_active_rays, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, p_first,
+                       ray_list, n_active, acc, depth, app_cnt, p_end);
     LM_CHECK_LAUNCH("k_active_rays");
     return LM_OK;
 }
 
-int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, const float *w_valid,
+int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
                         float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
                         uint32_t *app_idx, float *app_w, uint32_t *app_count, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, w_valid,
+    hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, p_first, w_valid,
                        weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count);
     LM_CHECK_LAUNCH("k_app_slots");
     return LM_OK;

@@ -363,7 +363,7 @@ __global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
                                                   const float *__restrict__ rays, const uint64_t *__restrict__ bitmap,
-                                                  const uint32_t *__restrict__ word_prefix,
+                                                  const uint32_t *__restrict__ p_first,
                                                   const uint32_t *__restrict__ ray_list,
                                                   const uint32_t *__restrict__ n_active_ptr, uint32_t *__restrict__ queue,
                                                   int act, float shift, float distance_scale, float weight_thres,
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
     uint64_t flat0 = 0;
     float ray[6] = {0, 0, 0, 0, 0, 0}, rp = 0.0f, Tr = 1.0f, acc = 0.0f, depth = 0.0f;
     BitWalk it;
-    it.bits = 0; it.w = it.w_last = 0; it.flat1 = 0; it.pos = 0; it.bitmap = bitmap; it.prefix = word_prefix;
+    it.bits = 0; it.w = it.w_last = 0; it.flat1 = 0; it.pos = 0; it.bitmap = bitmap; it.prefix = nullptr;
     while (true) {
         // quads without a ray take the next ones from the queue: one atomic per wave and round
         const bool need = !have && !done;
@@ -401,7 +401,7 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                     ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
                     rp = lm_ray_param(g, ray);
                     flat0 = (uint64_t)r * (uint64_t)S;
-                    it.start(bitmap, word_prefix, flat0, flat0 + S);
+                    it.start_at(bitmap, flat0, flat0 + S, p_first[r]);
                     p = it.pos;
                     Tr = 1.0f; acc = 0.0f; depth = 0.0f; cnt = 0;
                     have = true;
@@ -794,7 +794,7 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
 }
 
 // Density + transmittance march over the rays listed in ray_list (those with valid samples).
-int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *word_prefix,
+int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
                     const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st) {
     int dtype;
@@ -804,11 +804,11 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     const unsigned grid = (unsigned)lm_persistent_blocks(8);
     if (dtype == LM_F32)
         hipLaunchKernelGGL(k_march<float>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
-                           word_prefix, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
+                           p_first, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
                            m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
     else
         hipLaunchKernelGGL(k_march<__half>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
-                           word_prefix, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
+                           p_first, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
                            m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
     LM_CHECK_LAUNCH("k_march");
     return LM_OK;

@@ -72,6 +72,27 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *
 // same few cache lines (a wave of 64 samples along one ray touches 64 different ones), and the
 // per-ray work (slab test or hull distance) is done once per word instead of once per sample.
 // A workgroup covers 256 consecutive words = 4 of the 64-word groups k_scan_blocks counts.
+__device__ __forceinline__ uint64_t word_of_ray(const lm_geom &g, const float *__restrict__ rays, uint64_t r, unsigned j) {
+    float ray[6];
+    const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
+    const float2 a = rp2[0], b = rp2[1], c = rp2[2];
+    ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+    const float rp = lm_ray_param(g, ray);
+    const bool cells0 = g.vol && g.vol_dtype == LM_CELLS && g.vol_thre == 0.0f;
+    uint64_t bits = 0;
+#pragma unroll 4
+    for (int i = 0; i < 64; ++i) {
+        const float z = lm_sample_z(g, rp, (int)j * 64 + i);
+        float pt[3];
+        lm_point(ray, z, pt);
+        bool ok;
+        if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
+        else ok = lm_sample_valid(g, pt);
+        bits |= (uint64_t)ok << i;
+    }
+    return bits;
+}
+
 template <int WPR>
 __global__ __launch_bounds__(kBlock) void k_sample_cull_rays(lm_geom g, const float *__restrict__ rays, uint32_t N,
                                                              uint64_t nb, uint64_t *__restrict__ bitmap,
@@ -86,22 +107,7 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull_rays(lm_geom g, const fl
     const uint64_t r = (uint64_t)blockIdx.x * kRays + ray_local;
     uint64_t bits = 0;
     if (r < N) {
-        float ray[6];
-        const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
-        const float2 a = rp2[0], b = rp2[1], c = rp2[2];
-        ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
-        const float rp = lm_ray_param(g, ray);
-        const bool cells0 = g.vol && g.vol_dtype == LM_CELLS && g.vol_thre == 0.0f;
-#pragma unroll 4
-        for (int i = 0; i < 64; ++i) {
-            const float z = lm_sample_z(g, rp, (int)j * 64 + i);
-            float pt[3];
-            lm_point(ray, z, pt);
-            bool ok;
-            if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
-            else ok = lm_sample_valid(g, pt);
-            bits |= (uint64_t)ok << i;
-        }
+        bits = word_of_ray(g, rays, r, j);
         bitmap[r * WPR + j] = bits;
     }
     const uint32_t cnt = (uint32_t)__popcll(bits);
@@ -110,6 +116,61 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull_rays(lm_geom g, const fl
     if (threadIdx.x < 4) {
         const uint64_t bi = (uint64_t)blockIdx.x * 4 + threadIdx.x;
         if (bi < nb) block_count[bi] = s_cnt[threadIdx.x];
+    }
+}
+
+// The same words for the whole-chunk render, which needs no global order of the valid samples:
+// every ray gets a contiguous range of compact positions (p_first[r], wave prefix + one atomic on
+// n_valid), rays with valid samples are appended to the marching queue's list, the others get
+// their zero results here.  Replaces the scan, the per-word prefix and the list of active rays.
+template <int WPR>
+__global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const float *__restrict__ rays, uint32_t N,
+                                                            uint64_t *__restrict__ bitmap, uint32_t *__restrict__ p_first,
+                                                            uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
+                                                            uint32_t *__restrict__ n_valid, float *__restrict__ acc,
+                                                            float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
+                                                            uint32_t *__restrict__ p_end) {
+    __shared__ uint32_t s_cnt[kBlock];
+    const unsigned lane = lm_lane(), wave = threadIdx.x / LM_WAVE;
+    constexpr unsigned kRays = kBlock / WPR;
+    const unsigned j = wave % WPR;
+    const unsigned ray_local = (wave / WPR) * 64 + lane;
+    const uint64_t r = (uint64_t)blockIdx.x * kRays + ray_local;
+    uint64_t bits = 0;
+    if (r < N) {
+        bits = word_of_ray(g, rays, r, j);
+        bitmap[r * WPR + j] = bits;
+    }
+    s_cnt[ray_local * WPR + j] = (uint32_t)__popcll(bits);
+    __syncthreads();
+    if (j != 0) return;  // whole waves leave: j is wave-uniform
+    uint32_t cnt = 0;
+#pragma unroll
+    for (unsigned jj = 0; jj < (unsigned)WPR; ++jj) cnt += s_cnt[ray_local * WPR + jj];
+    uint32_t incl = cnt;
+#pragma unroll
+    for (int d = 1; d < LM_WAVE; d <<= 1) {
+        const uint32_t y = __shfl_up(incl, d);
+        if (lane >= (unsigned)d) incl += y;
+    }
+    const uint32_t total = __shfl(incl, LM_WAVE - 1);
+    uint32_t base = 0;
+    if (total) {
+        if (lane == 0) base = atomicAdd(n_valid, total);
+        base = __shfl(base, 0);
+    }
+    const bool any = cnt != 0;
+    if (r < N) {
+        const uint32_t first = base + incl - cnt;
+        p_first[r] = first;
+        if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
+    }
+    const uint64_t mask = __ballot(any);
+    if (mask) {
+        uint32_t slot = 0;
+        if (lane == 0) slot = atomicAdd(n_active, (uint32_t)__popcll(mask));
+        slot = __shfl(slot, 0);
+        if (any) ray_list[slot + lm_mbcnt(mask)] = (uint32_t)r;
     }
 }
 
@@ -342,5 +403,25 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
     hipLaunchKernelGGL(k_alpha_mask_pool, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, alpha, gx,
                        gy, gz, thres, volume, box, reinterpret_cast<unsigned long long *>(count));
     LM_CHECK_LAUNCH("k_alpha_mask_pool");
+    return LM_OK;
+}
+
+// Cull + per-ray set-up in one launch for the whole-chunk render; returns 1 when the sample count has
+// no such kernel (the caller then takes lm_sample_cull + the list kernel), 0 on success.
+int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
+                         uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
+                         uint32_t *app_cnt, uint32_t *p_end, hipStream_t st) {
+    const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
+    if (!(wpr == 1 || wpr == 2 || wpr == 4)) return 1;
+    LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
+    const unsigned groups = (unsigned)(((uint64_t)N * wpr + kBlock - 1) / kBlock);
+#define LM_CULL_SETUP(W_)                                                                                             \
+    hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3(groups), dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, bitmap, p_first, \
+                       ray_list, n_active, n_valid, acc, depth, app_cnt, p_end)
+    if (wpr == 1) LM_CULL_SETUP(1);
+    else if (wpr == 2) LM_CULL_SETUP(2);
+    else LM_CULL_SETUP(4);
+#undef LM_CULL_SETUP
+    LM_CHECK_LAUNCH("k_cull_rays_setup");
     return LM_OK;
 }
