@@ -85,6 +85,10 @@ def bench_frame(args, workload):
     chunk = min(args.chunk, N)
     while chunk * S >= 2**32:
         chunk //= 2
+    if not args.no_row_hint and W % 8 == 0:
+        # the rays are the frame's pixels row by row: tell the library, and cut chunks at whole bands of 8 rows
+        model.ray_row_length = W
+        chunk = max(8 * W, chunk // (8 * W) * (8 * W))
     n_chunks = (N + chunk - 1) // chunk
     rgb = torch.empty((N, 3), device=dev)
     depth = torch.empty((N,), device=dev)
@@ -162,7 +166,7 @@ def bench_frame(args, workload):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32" if args.mlp == "f32" else f"f32+{args.mlp}-mlp",
         "data": "synthetic",
-        "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "mlp": args.mlp,
+        "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "ray_row_hint": int(model.ray_row_length), "mlp": args.mlp,
                    "term_eps": args.term_eps, "valid_samples": n_valid, "marched_samples": n_marched, "app_samples": n_app},
         "frames_per_s": round(1e3 / ms_step, 3), "mpixel_per_s": round(mrays, 3),
         "gather_GBps": stages["density_march"]["GBps"],
@@ -324,6 +328,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=270)
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-row-hint", action="store_true", help="do not tell the library that rays are image rows")
     ap.add_argument("--calib", action="store_true", help="also run one 1 GiB device copy (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:

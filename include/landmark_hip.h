@@ -130,6 +130,13 @@ typedef struct lm_model {
     const void *mlp_packed; /* device copy of the buffer written by lm_mlp_pack */
     int32_t white_bg;
     float term_eps; /* > 0: stop marching a ray once transmittance < term_eps */
+    /* Hint: the chunk's rays are the pixels of an image stored row by row, ray_row of them per
+     * row (the chunk may start anywhere in a row).  lm_render then visits rays in 8 x 8 pixel
+     * tiles, so that rays handled together are neighbours in both directions and share more of
+     * the tables' cache lines.  Results and their order do not depend on it.  0 or not a
+     * multiple of 8: rays are visited in the order given. */
+    int32_t ray_row;
+    int32_t reserved_;
     /* Optional timing hooks: hipEvent_t handles created by the caller, or NULL.  lm_render
      * records events[0] before its first kernel and events[i] after stage i on `stream`
      * (LM_STAGE_*); it never waits on them. */

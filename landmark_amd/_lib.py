@@ -46,6 +46,7 @@ class LmModel(C.Structure):
         ("density", LmPlane * LM_MAX_PLANES), ("app", LmPlane * LM_MAX_PLANES),
         ("density_basis", C.c_void_p), ("act", C.c_int32), ("density_shift", C.c_float), ("distance_scale", C.c_float), ("weight_thres", C.c_float),
         ("mlp_prec", C.c_int32), ("mlp_packed", C.c_void_p), ("white_bg", C.c_int32), ("term_eps", C.c_float),
+        ("ray_row", C.c_int32), ("reserved_", C.c_int32),
         ("events", C.c_void_p * (LM_N_STAGES + 1)),
     ]
 

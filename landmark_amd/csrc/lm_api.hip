@@ -78,17 +78,18 @@ int lm_app_feat_supported(const lm_model *m);
 int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *feat, const float *rays,
                          const uint32_t *app_idx, const uint32_t *count, float *rgb, hipStream_t stream);
 int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
-                        const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream);
+                        const float *rgb, const float *acc, int white_bg, uint32_t row, float *rgb_map,
+                        hipStream_t stream);
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
 int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
                           uint32_t *ray_list, uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt,
-                          uint32_t *p_end, hipStream_t stream);
+                          uint32_t *p_end, uint32_t row, hipStream_t stream);
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
-                         uint32_t *app_cnt, uint32_t *p_end, hipStream_t st);
+                         uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st);
 int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
                         float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
-                        uint32_t *app_idx, float *app_w, uint32_t *app_count, hipStream_t stream);
+                        uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, hipStream_t stream);
 int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
                     const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st);
@@ -188,18 +189,20 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     auto mark = [&](int i) {
         if (m->events[i]) (void)hipEventRecord((hipEvent_t)m->events[i], st);
     };
+    LM_REQUIRE(m->ray_row >= 0, "negative ray_row");
+    const uint32_t row = m->ray_row % 8 == 0 ? (uint32_t)m->ray_row : 0u;  // tiles of 8 x 8 pixels need whole tiles per row
     mark(0);
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
     // sample counts of 64, 128 or 256: one launch decides the samples and sets the rays up; otherwise the
     // stage-level cull (scan + per-word prefix) followed by the list kernel
     int rc_setup = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE,
-                                        cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, st);
+                                        cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, st);
     if (rc_setup < 0) return rc_setup;
     if (rc_setup > 0) {
         if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, nullptr, cnt, nullptr, w.cull_scratch, st))
             return rc;
         if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE,
-                                           w.acc, depth_map, w.app_cnt, w.p_end, st))
+                                           w.acc, depth_map, w.app_cnt, w.p_end, row, st))
             return rc;
     }
     mark(LM_STAGE_CULL);
@@ -208,7 +211,7 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
         return rc;
     mark(LM_STAGE_DENSITY);
     if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.p_first, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
-                                     w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, st))
+                                     w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, row, st))
         return rc;
     mark(LM_STAGE_WEIGHTS);
     if (fused) {
@@ -222,7 +225,7 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     if (int rc = lm_launch_app_colour(m->mlp_prec, m->mlp_packed, K, S, w.feat, rays, w.app_idx, cnt + LM_STAT_N_APP, w.rgb, st))
         return rc;
     mark(LM_STAGE_COLOUR);
-    if (int rc = lm_launch_composite(N, w.app_first, w.app_cnt, w.app_w, w.rgb, w.acc, m->white_bg, rgb_map, st)) return rc;
+    if (int rc = lm_launch_composite(N, w.app_first, w.app_cnt, w.app_w, w.rgb, w.acc, m->white_bg, row, rgb_map, st)) return rc;
     mark(LM_STAGE_COMPOSITE);
     return LM_OK;
 }

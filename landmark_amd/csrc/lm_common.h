@@ -236,6 +236,19 @@ __device__ __forceinline__ unsigned lm_mbcnt(uint64_t mask) {  // set bits of ma
     return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
 
+// Visiting order of the whole-chunk render when the rays are image rows of length W (a
+// multiple of 8): position o -> ray index, 8 x 8 pixel tiles inside bands of 8 rows; the rays
+// behind the last full band keep their order.  A bijection on [0, N).
+__device__ __forceinline__ uint32_t lm_ray_order(uint32_t o, uint32_t N, uint32_t W) {
+    if (W == 0) return o;
+    const uint32_t band = 8u * W;
+    const uint32_t full = (N / band) * band;
+    if (o >= full) return o;
+    const uint32_t b = o / band, t = o - b * band;
+    const uint32_t tile = t >> 6, in = t & 63u;
+    return b * band + (in >> 3) * W + tile * 8u + (in & 7u);
+}
+
 // Iterates the set bits of the sample bitmap in [flat0, flat1): the valid samples of one ray.
 struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
     const uint64_t *bitmap;

@@ -105,10 +105,11 @@ __global__ __launch_bounds__(kBlock) void k_weights(lm_geom g, const float *__re
 __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t *__restrict__ app_first,
                                                       const uint32_t *__restrict__ app_cnt,
                                                       const float *__restrict__ app_w, const float *__restrict__ rgb,
-                                                      const float *__restrict__ acc, int white_bg,
+                                                      const float *__restrict__ acc, int white_bg, uint32_t row,
                                                       float *__restrict__ rgb_map) {
-    const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (r >= N) return;
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (o >= N) return;
+    const uint64_t r = lm_ray_order((uint32_t)o, (uint32_t)N, row);
     float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f;
     const uint32_t first = app_first[r], n = app_cnt[r];
     for (uint32_t i = 0; i < n; ++i) {
@@ -132,9 +133,11 @@ __global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const
                                                         uint32_t *__restrict__ p_first,
                                                         uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
                                                         float *__restrict__ acc, float *__restrict__ depth,
-                                                        uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end) {
+                                                        uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end,
+                                                        uint32_t row) {
     const unsigned lane = lm_lane();
-    const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t r = o < N ? lm_ray_order((uint32_t)o, (uint32_t)N, row) : o;
     bool any = false;
     if (r < N) {
         BitWalk it;
@@ -161,9 +164,11 @@ __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const u
                                                       const uint32_t *__restrict__ app_cnt,
                                                       const uint32_t *__restrict__ p_end,
                                                       uint32_t *__restrict__ app_first, uint32_t *__restrict__ app_idx,
-                                                      float *__restrict__ app_w, uint32_t *__restrict__ app_count) {
+                                                      float *__restrict__ app_w, uint32_t *__restrict__ app_count,
+                                                      uint32_t row) {
     const unsigned lane = lm_lane();
-    const uint64_t r = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint64_t r = o < N ? lm_ray_order((uint32_t)o, (uint32_t)N, row) : o;
     const uint32_t cnt = r < N ? app_cnt[r] : 0;
     uint32_t incl = cnt;
 #pragma unroll
@@ -224,11 +229,12 @@ extern "C" int lm_weights(const lm_geom *geom, const float *rays, int64_t N, con
 }
 
 int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
-                        const float *rgb, const float *acc, int white_bg, float *rgb_map, hipStream_t stream) {
+                        const float *rgb, const float *acc, int white_bg, uint32_t row, float *rgb_map,
+                        hipStream_t stream) {
     if (N == 0) return LM_OK;
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(k_composite, dim3(grid), dim3(kBlock), 0, stream, (uint64_t)N, app_first, app_cnt, app_w, rgb, acc,
-                       white_bg, rgb_map);
+                       white_bg, row, rgb_map);
     LM_CHECK_LAUNCH("k_composite");
     return LM_OK;
 }
@@ -241,20 +247,20 @@ int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
 
 int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
                           uint32_t *ray_list, uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt,
-                          uint32_t *p_end, hipStream_t stream) {
+                          uint32_t *p_end, uint32_t row, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(k_active_rays, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, p_first,
-                       ray_list, n_active, acc, depth, app_cnt, p_end);
+                       ray_list, n_active, acc, depth, app_cnt, p_end, row);
     LM_CHECK_LAUNCH("k_active_rays");
     return LM_OK;
 }
 
 int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
                         float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
-                        uint32_t *app_idx, float *app_w, uint32_t *app_count, hipStream_t stream) {
+                        uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, p_first, w_valid,
-                       weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count);
+                       weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count, row);
     LM_CHECK_LAUNCH("k_app_slots");
     return LM_OK;
 }

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull_rays(lm_geom g, const fl
 // their zero results here.  Replaces the scan, the per-word prefix and the list of active rays.
 template <int WPR>
 __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const float *__restrict__ rays, uint32_t N,
-                                                            uint64_t *__restrict__ bitmap, uint32_t *__restrict__ p_first,
+                                                            uint32_t row, uint64_t *__restrict__ bitmap, uint32_t *__restrict__ p_first,
                                                             uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
                                                             uint32_t *__restrict__ n_valid, float *__restrict__ acc,
                                                             float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
@@ -135,7 +135,8 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
     constexpr unsigned kRays = kBlock / WPR;
     const unsigned j = wave % WPR;
     const unsigned ray_local = (wave / WPR) * 64 + lane;
-    const uint64_t r = (uint64_t)blockIdx.x * kRays + ray_local;
+    const uint64_t o = (uint64_t)blockIdx.x * kRays + ray_local;  // position in the visiting order
+    const uint64_t r = o < N ? lm_ray_order((uint32_t)o, N, row) : o;
     uint64_t bits = 0;
     if (r < N) {
         bits = word_of_ray(g, rays, r, j);
@@ -410,13 +411,13 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
 // no such kernel (the caller then takes lm_sample_cull + the list kernel), 0 on success.
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
-                         uint32_t *app_cnt, uint32_t *p_end, hipStream_t st) {
+                         uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st) {
     const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
     if (!(wpr == 1 || wpr == 2 || wpr == 4)) return 1;
     LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
     const unsigned groups = (unsigned)(((uint64_t)N * wpr + kBlock - 1) / kBlock);
 #define LM_CULL_SETUP(W_)                                                                                             \
-    hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3(groups), dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, bitmap, p_first, \
+    hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3(groups), dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, \
                        ray_list, n_active, n_valid, acc, depth, app_cnt, p_end)
     if (wpr == 1) LM_CULL_SETUP(1);
     else if (wpr == 2) LM_CULL_SETUP(2);

@@ -54,6 +54,9 @@ class GridNeRFHIP:
         self.p = params
         self.mlp_precision = mlp_precision
         self.term_eps = float(term_eps)
+        # set by callers that render images: rays arrive row by row, this many per row (0 = unknown); lets the
+        # kernels visit rays in 8 x 8 pixel tiles.  Results do not depend on it.
+        self.ray_row_length = 0
         if params.app_dim != 27 or params.view_pe != 2 or params.fea_pe != 2 or params.featureC != 128:
             raise L.LandmarkError("colour network shape must be app_dim 27, view_pe = fea_pe = 2, featureC 128")
         if params.fea2denseAct not in ("softplus", "relu"):
@@ -276,6 +279,7 @@ class GridNeRFHIP:
         m.mlp_prec, m.mlp_packed = prec, packed.data_ptr()
         m.white_bg = int(bool(white_bg))
         m.term_eps = self.term_eps
+        m.ray_row = int(self.ray_row_length)
         return m
 
     def _samples_for(self, N_samples: int) -> int:

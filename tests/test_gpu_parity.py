@@ -367,6 +367,21 @@ def test_chunk_drivers(gpu_lib):
         m(rays, is_train=True)
 
 
+@pytest.mark.parametrize("S,width", [(128, 96), (64, 40), (100, 96), (128, 50)])
+def test_row_length_hint_changes_nothing(gpu_lib, S, width):
+    """ray_row only changes the order in which rays are visited (8 x 8 pixel tiles): bit-identical output, for
+    chunks that start mid-row and end mid-band, sample counts with and without the one-launch cull, and a row
+    length that is not a multiple of 8 (ignored)."""
+    p = _scene(opt=1, S=S, thre=0.0)
+    rays = scenes.pinhole_rays(width, 61, 70.0, scenes.sphere_pose(2.5, 9))[37:]
+    m = _model(p)
+    a, _ = m(rays)
+    m.ray_row_length = width
+    b, _ = m(rays)
+    assert torch.equal(a["rgb_map"], b["rgb_map"]) and torch.equal(a["depth_map"], b["depth_map"])
+    assert a["rgb_map"].min() < 0.99
+
+
 def test_early_termination_bounds(gpu_lib):
     p = _scene(S=128)
     rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
