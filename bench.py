@@ -321,7 +321,7 @@ def main():
     ap.add_argument("--term-eps", default="auto",
                     help="ray termination threshold on the transmittance; 'auto' = 1e-4 / far, the largest value that "
                          "keeps rgb and depth within 1e-4 of the unterminated render; 0 = never terminate")
-    ap.add_argument("--chunk", type=int, default=262144)
+    ap.add_argument("--chunk", type=int, default=1048576)
     ap.add_argument("--queries", type=int, default=1 << 24)
     ap.add_argument("--rows", type=int, default=1 << 23)
     ap.add_argument("--coherent", action="store_true")

@@ -144,9 +144,10 @@ typedef struct lm_model {
 } lm_model;
 
 /* Counters written by lm_render (device memory, 8 x uint32). */
-/* N_ACTIVE: rays with at least one valid sample; QUEUE: internal work-queue cursor;
- * N_MARCHED: valid samples whose density was gathered (< N_VALID with early termination) */
-enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_ACTIVE = 2, LM_STAT_QUEUE = 3, LM_STAT_N_MARCHED = 4, LM_STAT_WORDS = 8 };
+/* N_MARCHED: valid samples whose density was gathered (< N_VALID with early termination);
+ * QUEUE: internal work-queue cursor; BINS..BINS+3: rays with valid samples, by how many they have
+ * (>= 64, >= 32, >= 12, fewer): the marching queue hands out the long rays first. */
+enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_MARCHED = 2, LM_STAT_QUEUE = 3, LM_STAT_BINS = 4, LM_STAT_WORDS = 8 };
 
 int lm_abi_version(void);
 const char *lm_last_error(void);

@@ -91,7 +91,7 @@ int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t
                         float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
                         uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, hipStream_t stream);
 int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
-                    const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
+                    const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid, float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st);
 int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
                     float *feat, hipStream_t st);
@@ -136,7 +136,7 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products)
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
     w.p_first = (uint32_t *)take((uint64_t)N * 4);
     w.p_end = (uint32_t *)take((uint64_t)N * 4);
-    w.ray_list = (uint32_t *)take((uint64_t)N * 4);
+    w.ray_list = (uint32_t *)take((uint64_t)N * 4 * LM_RAY_BINS);  // one list per bin of the marching queue
     w.app_idx = (uint32_t *)take(cap * 4);
     w.app_w = (float *)take(cap * 4);
     w.rgb = (float *)take(cap * 12);
@@ -195,18 +195,18 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
     // sample counts of 64, 128 or 256: one launch decides the samples and sets the rays up; otherwise the
     // stage-level cull (scan + per-word prefix) followed by the list kernel
-    int rc_setup = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE,
+    int rc_setup = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
                                         cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, st);
     if (rc_setup < 0) return rc_setup;
     if (rc_setup > 0) {
         if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, nullptr, cnt, nullptr, w.cull_scratch, st))
             return rc;
-        if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE,
+        if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
                                            w.acc, depth_map, w.app_cnt, w.p_end, row, st))
             return rc;
     }
     mark(LM_STAGE_CULL);
-    if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_N_ACTIVE, cnt + LM_STAT_QUEUE,
+    if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS, (uint32_t)N, cnt + LM_STAT_QUEUE,
                                  w.w_valid, w.acc, depth_map, w.app_cnt, w.p_end, cnt + LM_STAT_N_MARCHED, st))
         return rc;
     mark(LM_STAGE_DENSITY);

@@ -236,6 +236,30 @@ __device__ __forceinline__ unsigned lm_mbcnt(uint64_t mask) {  // set bits of ma
     return __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u));
 }
 
+// Rays waiting for the marching kernel are kept in four lists by their number of valid samples
+// (an upper bound of the work they are), list b at ray_list + b * N, so that the queue can hand
+// out the long ones first: a launch then does not end with a few long rays marching alone.
+#define LM_RAY_BINS 4
+__device__ __forceinline__ int lm_ray_bin(uint32_t n_valid) {
+    return n_valid >= 64u ? 0 : (n_valid >= 32u ? 1 : (n_valid >= 12u ? 2 : 3));
+}
+// append the lanes with `mine` set to their lists (one atomic per wave and non-empty list)
+__device__ __forceinline__ void lm_ray_enqueue(bool mine, int bin, uint32_t r, uint32_t *ray_list, uint32_t N,
+                                               uint32_t *bins) {
+#pragma unroll
+    for (int b = 0; b < LM_RAY_BINS; ++b) {
+        const uint64_t mask = __ballot(mine && bin == b);
+        if (mask == 0) continue;
+        uint32_t slot = 0;
+        const int first = __ffsll((unsigned long long)mask) - 1;
+        if ((int)__lane_id() == first) slot = atomicAdd(bins + b, (uint32_t)__popcll(mask));
+        slot = __shfl(slot, first);
+        if (mine && bin == b)
+            ray_list[(size_t)b * N + slot +
+                     __builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)mask, 0u))] = r;
+    }
+}
+
 // Visiting order of the whole-chunk render when the rays are image rows of length W (a
 // multiple of 8): position o -> ray index, 8 x 8 pixel tiles inside bands of 8 rows; the rays
 // behind the last full band keep their order.  A bijection on [0, N).

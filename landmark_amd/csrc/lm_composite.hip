@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
 __global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
                                                         const uint32_t *__restrict__ word_prefix,
                                                         uint32_t *__restrict__ p_first,
-                                                        uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
+                                                        uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
                                                         float *__restrict__ acc, float *__restrict__ depth,
                                                         uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end,
                                                         uint32_t row) {
@@ -147,13 +147,7 @@ __global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const
         any = it.next(flat);
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = it.pos; }
     }
-    const uint64_t mask = __ballot(any);
-    if (mask) {
-        uint32_t base = 0;
-        if (lane == 0) base = atomicAdd(n_active, (uint32_t)__popcll(mask));
-        base = __shfl(base, 0);
-        if (any) ray_list[base + lm_mbcnt(mask)] = (uint32_t)r;
-    }
+    lm_ray_enqueue(any, 0, (uint32_t)r, ray_list, (uint32_t)N, bins);  // one list: the counts are not known here
 }
 
 // Appearance list from stored weights: a contiguous slot range per ray (wave prefix + one
@@ -246,11 +240,11 @@ int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
 }
 
 int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
-                          uint32_t *ray_list, uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt,
+                          uint32_t *ray_list, uint32_t *bins, float *acc, float *depth, uint32_t *app_cnt,
                           uint32_t *p_end, uint32_t row, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(k_active_rays, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, p_first,
-                       ray_list, n_active, acc, depth, app_cnt, p_end, row);
+                       ray_list, bins, acc, depth, app_cnt, p_end, row);
     LM_CHECK_LAUNCH("k_active_rays");
     return LM_OK;
 }

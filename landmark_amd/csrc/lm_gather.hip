@@ -169,6 +169,81 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
     return den_w ? fmaxf(sum, 0.0f) : sum;
 }
 
+// The loads of plane_products and the arithmetic on what they return, as two steps, for callers
+// that want several footprints' loads in flight before the first use.
+template <typename T> struct Footprint {
+    float a[Vec<T>::V], b[Vec<T>::V], c[Vec<T>::V], d[Vec<T>::V], l0[Vec<T>::V], l1[Vec<T>::V];
+};
+template <typename T>
+__device__ __forceinline__ void footprint_load(const lm_plane &pl, const Taps2 &t2, const Taps1 &t1, int c, Footprint<T> &f) {
+    const T *P = reinterpret_cast<const T *>(pl.plane);
+    const T *Ln = reinterpret_cast<const T *>(pl.line);
+    Vec<T>::load(P + t2.o00 + c, f.a);
+    Vec<T>::load(P + t2.o01 + c, f.b);
+    Vec<T>::load(P + t2.o10 + c, f.c);
+    Vec<T>::load(P + t2.o11 + c, f.d);
+    Vec<T>::load(Ln + t1.o0 + c, f.l0);
+    Vec<T>::load(Ln + t1.o1 + c, f.l1);
+}
+template <typename T>
+__device__ __forceinline__ void footprint_products(const Footprint<T> &f, const Taps2 &t2, const Taps1 &t1, float *prod) {
+#pragma unroll
+    for (int i = 0; i < Vec<T>::V; ++i) {
+        float pv = f.a[i] * t2.w00;
+        pv = fmaf(f.b[i], t2.w01, pv);
+        pv = fmaf(f.c[i], t2.w10, pv);
+        pv = fmaf(f.d[i], t2.w11, pv);
+        const float lv = fmaf(f.l1[i], t1.w1, f.l0[i] * t1.w0);
+        prod[i] = pv * lv;
+    }
+}
+
+// Two samples at once (the marching kernel's look-ahead): the loads of both are issued before
+// either is used, so a ray's chain of dependent memory round trips is half as long.  Same
+// operations per sample as density_sum, hence the same bits.
+template <typename T>
+__device__ __forceinline__ void density_sum2(const PlaneSet &ps, const float *qa, const float *qb, unsigned qlane,
+                                             const float *__restrict__ den_w, float &out_a, float &out_b) {
+    constexpr int V = Vec<T>::V;
+    float sa = 0.0f, sb = 0.0f;
+    int col = 0;
+    for (int k = 0; k < ps.n; ++k) {
+        const lm_plane &pl = ps.p[k];
+        Taps2 a2 = plane_taps(pl, pick(qa, pl.ax0), pick(qa, pl.ax1));
+        Taps1 a1 = line_taps(pl, pick(qa, pl.axl));
+        block_taps(pl, ps.nblk, qa, a2, a1);
+        Taps2 b2 = plane_taps(pl, pick(qb, pl.ax0), pick(qb, pl.ax1));
+        Taps1 b1 = line_taps(pl, pick(qb, pl.axl));
+        block_taps(pl, ps.nblk, qb, b2, b1);
+        for (int c = V * qlane; c < pl.C; c += V * kQuad) {
+            Footprint<T> fa, fb;
+            footprint_load<T>(pl, a2, a1, c, fa);
+            footprint_load<T>(pl, b2, b1, c, fb);
+            // keep the twelve loads ahead of the first use
+            __builtin_amdgcn_sched_barrier(0);
+            float pa[V], pb[V];
+            footprint_products<T>(fa, a2, a1, pa);
+            footprint_products<T>(fb, b2, b1, pb);
+            if (den_w) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) sa = fmaf(den_w[col + c + i], pa[i], sa);
+#pragma unroll
+                for (int i = 0; i < V; ++i) sb = fmaf(den_w[col + c + i], pb[i], sb);
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; ++i) sa += pa[i];
+#pragma unroll
+                for (int i = 0; i < V; ++i) sb += pb[i];
+            }
+        }
+        col += pl.C;
+    }
+    sa += __shfl_xor(sa, 1); sb += __shfl_xor(sb, 1);
+    sa += __shfl_xor(sa, 2); sb += __shfl_xor(sb, 2);
+    out_a = den_w ? fmaxf(sa, 0.0f) : sa;
+    out_b = den_w ? fmaxf(sb, 0.0f) : sb;
+}
+
 // Same sum with a compile-time channel count shared by all planes: the channel groups of a
 // plane are unrolled, so a lane has 6 * C / (4 V) independent loads in flight per plane
 // instead of 6 (wide planes, e.g. the 64-channel isolated-gather configuration).
@@ -365,7 +440,8 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                                                   const float *__restrict__ rays, const uint64_t *__restrict__ bitmap,
                                                   const uint32_t *__restrict__ p_first,
                                                   const uint32_t *__restrict__ ray_list,
-                                                  const uint32_t *__restrict__ n_active_ptr, uint32_t *__restrict__ queue,
+                                                  const uint32_t *__restrict__ bins, uint32_t n_rays,
+                                                  uint32_t *__restrict__ queue,
                                                   int act, float shift, float distance_scale, float weight_thres,
                                                   float term_eps, float *__restrict__ w_valid,
                                                   float *__restrict__ acc_out, float *__restrict__ depth_out,
@@ -373,7 +449,8 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                                                   uint32_t *__restrict__ n_marched) {
     const unsigned lane = lm_lane(), qlane = lane & 3u, leader = lane & ~3u;
     uint32_t marched = 0;  // samples whose density this lane's quad gathered (statistics)
-    const uint32_t n_active = *n_active_ptr;
+    // cumulative sizes of the four ray lists (long rays first)
+    const uint32_t end0 = bins[0], end1 = end0 + bins[1], end2 = end1 + bins[2], n_active = end2 + bins[3];
     const int S = g.S;
     bool have = false, done = false;
     uint32_t r = 0, p = 0, cnt = 0;
@@ -395,7 +472,10 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                 if (idx >= n_active) {
                     done = true;
                 } else {
-                    r = ray_list[idx];
+                    r = idx < end0   ? ray_list[idx]
+                        : idx < end1 ? ray_list[(size_t)n_rays + (idx - end0)]
+                        : idx < end2 ? ray_list[2 * (size_t)n_rays + (idx - end1)]
+                                     : ray_list[3 * (size_t)n_rays + (idx - end2)];
                     const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
                     const float2 a = rp2[0], b = rp2[1], c = rp2[2];
                     ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
@@ -410,28 +490,42 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
         }
         if (!__any(have)) break;
         if (have) {
-            uint64_t flat;
-            bool finish = !it.next(flat);
+            // up to two samples per round: both densities are gathered together, the weights follow in order
+            uint64_t flat_a, flat_b = 0;
+            bool finish = !it.next(flat_a);
             if (!finish) {
-                const int s = (int)(flat - flat0);
-                const float z = lm_sample_z(g, rp, s);
-                float pt[3], q[4];
-                lm_point(ray, z, pt);
-                lm_normalise(g, pt, q);
-                q[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q) : 0);
-                const float sig = activate(density_sum<T>(ps, q, qlane, den_w), act, shift);
-                const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
-                const float d2 = dist * distance_scale;
-                const float alpha = 1.0f - expf(-sig * d2);
-                const float wgt = alpha * Tr;
-                Tr = Tr * ((1.0f - alpha) + 1e-10f);
-                if (qlane == 0) w_valid[p] = wgt;
-                acc += wgt;
-                depth += wgt * z;
-                cnt += wgt > weight_thres;
-                ++p;
-                ++marched;
-                finish = term_eps > 0.0f && Tr < term_eps;
+                const bool two = it.next(flat_b);
+                const int s_a = (int)(flat_a - flat0), s_b = two ? (int)(flat_b - flat0) : s_a;
+                const float z_a = lm_sample_z(g, rp, s_a), z_b = lm_sample_z(g, rp, s_b);
+                float pt[3], q_a[4], q_b[4];
+                lm_point(ray, z_a, pt);
+                lm_normalise(g, pt, q_a);
+                q_a[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q_a) : 0);
+                lm_point(ray, z_b, pt);
+                lm_normalise(g, pt, q_b);
+                q_b[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q_b) : 0);
+                float f_a, f_b;
+                density_sum2<T>(ps, q_a, q_b, qlane, den_w, f_a, f_b);
+                marched += two ? 2u : 1u;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    if (h == 1 && (!two || finish)) break;
+                    const int s = h ? s_b : s_a;
+                    const float z = h ? z_b : z_a;
+                    const float sig = activate(h ? f_b : f_a, act, shift);
+                    const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
+                    const float d2 = dist * distance_scale;
+                    const float alpha = 1.0f - expf(-sig * d2);
+                    const float wgt = alpha * Tr;
+                    Tr = Tr * ((1.0f - alpha) + 1e-10f);
+                    if (qlane == 0) w_valid[p] = wgt;
+                    acc += wgt;
+                    depth += wgt * z;
+                    cnt += wgt > weight_thres;
+                    ++p;
+                    finish = term_eps > 0.0f && Tr < term_eps;
+                }
+                if (!two) finish = true;  // the ray's last sample
             }
             if (finish) {
                 if (qlane == 0) {
@@ -795,20 +889,21 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
 
 // Density + transmittance march over the rays listed in ray_list (those with valid samples).
 int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
-                    const uint32_t *ray_list, const uint32_t *n_active, uint32_t *queue, float *w_valid, float *acc,
+                    const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid,
+                    float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st) {
     int dtype;
     if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
     LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
     const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
-    const unsigned grid = (unsigned)lm_persistent_blocks(8);
+    const unsigned grid = (unsigned)lm_persistent_blocks(4);
     if (dtype == LM_F32)
         hipLaunchKernelGGL(k_march<float>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
-                           p_first, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
+                           p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,
                            m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
     else
         hipLaunchKernelGGL(k_march<__half>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
-                           p_first, ray_list, n_active, queue, m->act, m->density_shift, m->distance_scale,
+                           p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,
                            m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
     LM_CHECK_LAUNCH("k_march");
     return LM_OK;

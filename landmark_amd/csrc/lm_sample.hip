@@ -121,12 +121,12 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull_rays(lm_geom g, const fl
 
 // The same words for the whole-chunk render, which needs no global order of the valid samples:
 // every ray gets a contiguous range of compact positions (p_first[r], wave prefix + one atomic on
-// n_valid), rays with valid samples are appended to the marching queue's list, the others get
+// n_valid), rays with valid samples are appended to the marching queue's lists, the others get
 // their zero results here.  Replaces the scan, the per-word prefix and the list of active rays.
 template <int WPR>
 __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const float *__restrict__ rays, uint32_t N,
                                                             uint32_t row, uint64_t *__restrict__ bitmap, uint32_t *__restrict__ p_first,
-                                                            uint32_t *__restrict__ ray_list, uint32_t *__restrict__ n_active,
+                                                            uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
                                                             uint32_t *__restrict__ n_valid, float *__restrict__ acc,
                                                             float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
                                                             uint32_t *__restrict__ p_end) {
@@ -166,13 +166,7 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
         p_first[r] = first;
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
     }
-    const uint64_t mask = __ballot(any);
-    if (mask) {
-        uint32_t slot = 0;
-        if (lane == 0) slot = atomicAdd(n_active, (uint32_t)__popcll(mask));
-        slot = __shfl(slot, 0);
-        if (any) ray_list[slot + lm_mbcnt(mask)] = (uint32_t)r;
-    }
+    lm_ray_enqueue(any && r < N, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
 }
 
 // exclusive scan of n counts by one workgroup of 1024 threads; total -> *total_out
@@ -410,7 +404,7 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
 // Cull + per-ray set-up in one launch for the whole-chunk render; returns 1 when the sample count has
 // no such kernel (the caller then takes lm_sample_cull + the list kernel), 0 on success.
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
-                         uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
+                         uint32_t *ray_list, uint32_t *bins, uint32_t *n_valid, float *acc, float *depth,
                          uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st) {
     const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
     if (!(wpr == 1 || wpr == 2 || wpr == 4)) return 1;
@@ -418,7 +412,7 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
     const unsigned groups = (unsigned)(((uint64_t)N * wpr + kBlock - 1) / kBlock);
 #define LM_CULL_SETUP(W_)                                                                                             \
     hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3(groups), dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, \
-                       ray_list, n_active, n_valid, acc, depth, app_cnt, p_end)
+                       ray_list, bins, n_valid, acc, depth, app_cnt, p_end)
     if (wpr == 1) LM_CULL_SETUP(1);
     else if (wpr == 2) LM_CULL_SETUP(2);
     else LM_CULL_SETUP(4);
