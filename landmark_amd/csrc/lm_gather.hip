@@ -587,6 +587,7 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
     constexpr int NP = Mm::NP;
     constexpr int V = Vec<T>::V;
     constexpr int C = 16 * NU, ROW = C + 4;
+    constexpr int NG = (C + V * kQuad - 1) / (V * kQuad);  // 16-byte loads per lane, corner and plane
     static_assert(Mm::G == 8 && Mm::CW == 8, "the fused gather feeds 16-bit MFMAs");
     extern __shared__ __align__(16) char lds[];
     const size_t basis_bytes = (size_t)32 * K * sizeof(typename Mm::elem) * NP;
@@ -617,24 +618,49 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
         int t = 0;  // running MFMA step over the concatenated channels
-        for (int k = 0; k < ps.n; ++k) {
+        // Both samples' footprints of a plane are loaded with every load issued before the first use
+        // (one memory round trip per plane), and the loads of plane k + 1 are issued before the
+        // matrix step of plane k, which then runs under their latency.
+        Taps2 t2[2];
+        Taps1 t1[2];
+        Footprint<T> fp[2][NG];
+        auto issue = [&](int k) {
             const lm_plane &pl = ps.p[k];
 #pragma unroll
             for (int pass = 0; pass < 2; ++pass) {
                 const float *q = pass ? q1 : q0;
-                Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-                Taps1 t1 = line_taps(pl, pick(q, pl.axl));
-                block_taps(pl, ps.nblk, q, t2, t1);
+                t2[pass] = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+                t1[pass] = line_taps(pl, pick(q, pl.axl));
+                block_taps(pl, ps.nblk, q, t2[pass], t1[pass]);
+            }
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass)
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi) {
+                    const int c = V * (int)qlane + gi * V * kQuad;
+                    if (c < C) footprint_load<T>(pl, t2[pass], t1[pass], c, fp[pass][gi]);
+                }
+        };
+        issue(0);
+        for (int k = 0; k < ps.n; ++k) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
                 float *row = tile + (pass * 16 + gs) * ROW;
 #pragma unroll
-                for (int c = V * (int)qlane; c < C; c += V * kQuad) {
+                for (int gi = 0; gi < NG; ++gi) {
+                    const int c = V * (int)qlane + gi * V * kQuad;
+                    if (c >= C) continue;
                     float prod[V];
-                    plane_products<T>(pl, t2, t1, c, prod);
+                    footprint_products<T>(fp[pass][gi], t2[pass], t1[pass], prod);
 #pragma unroll
                     for (int i = 0; i < V; i += 4)
                         *reinterpret_cast<float4 *>(row + c + i) = make_float4(prod[i], prod[i + 1], prod[i + 2], prod[i + 3]);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (k + 1 < ps.n) issue(k + 1);
+            __builtin_amdgcn_sched_barrier(0);
             // LDS operations of one wave complete in order; the fence only pins the compiler
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
