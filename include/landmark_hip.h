@@ -46,7 +46,9 @@ enum { LM_ACT_SOFTPLUS = 0, LM_ACT_RELU = 1 };     /* fea2denseAct */
 /* arithmetic of the colour network's and basis_mat's matrix products (accumulation is
  * always fp32).  F16X2 splits every operand into two fp16 parts (x = hi + lo) and forms
  * hi*hi + lo*hi + hi*lo with three fp16 MFMAs: about 21 mantissa bits, for results that
- * must stay within 1e-4 of an fp32 evaluation. */
+ * must stay within 1e-4 of an fp32 evaluation.  F16 and F16X2 carry features, plane x line
+ * products and hidden activations as fp16 numbers: their magnitudes must stay below 65504
+ * (F32 and BF16 have the full float range). */
 enum { LM_MLP_F32 = 0, LM_MLP_F16 = 1, LM_MLP_BF16 = 2, LM_MLP_F16X2 = 3 };
 
 /* One feature plane with its line (one entry of density_plane/density_line or

@@ -41,16 +41,28 @@
 #ifndef LM_MLP_NCB
 #define LM_MLP_NCB 2
 #endif
+// split-fp16 mode: eight waves with one column block each (two waves per SIMD, so that one wave's
+// encoding and conversions run under the other's MFMAs) beat four waves with two (2.37 -> 2.15 ms
+// on 2^23 rows) although 87 registers spill
+#ifndef LM_MLPX2_THREADS
+#define LM_MLPX2_THREADS 512
+#endif
+#ifndef LM_MLPX2_NCB
+#define LM_MLPX2_NCB 1
+#endif
 
 namespace {
 
 using namespace lm_mma;
 
-// 16-bit modes: 8 waves per workgroup (two per SIMD, 256 registers each); the split and fp32
-// modes need the full register file of a SIMD per wave
+// 16-bit and split modes: 8 waves per workgroup (two per SIMD, 256 registers each); the fp32
+// mode needs the full register file of a SIMD per wave
 template <int PREC> struct MlpBlock {
-    static constexpr int N = (PREC == LM_MLP_F16 || PREC == LM_MLP_BF16) ? LM_MLP16_THREADS : 256;
-    static constexpr int NCB = PREC == LM_MLP_F32 ? 1 : LM_MLP_NCB;  // 32-sample column blocks per wave
+    static constexpr int N = (PREC == LM_MLP_F16 || PREC == LM_MLP_BF16) ? LM_MLP16_THREADS
+                             : PREC == LM_MLP_F16X2                        ? LM_MLPX2_THREADS
+                                                                           : 256;
+    // 32-sample column blocks per wave
+    static constexpr int NCB = PREC == LM_MLP_F32 ? 1 : (PREC == LM_MLP_F16X2 ? LM_MLPX2_NCB : LM_MLP_NCB);
 };
 
 // ---- host-side packing ----------------------------------------------------------------------
@@ -143,13 +155,11 @@ __device__ __forceinline__ floatx16 load_bias(const float *b, int idx) {
     return a;
 }
 
-// sin and cos of x to float rounding for |x| < 8192 (three-constant Cody-Waite reduction by
-// pi/2, then the minimax polynomials on [-pi/4, pi/4]); library routines beyond that.
+// sin and cos of x to float rounding for |x| <= 8192 (three-constant Cody-Waite reduction by
+// pi/2, then the minimax polynomials on [-pi/4, pi/4]); callers redo larger arguments with the
+// library routines (kSincosMax), outside their hot loop.
+constexpr float kSincosMax = 8192.0f;
 __device__ __forceinline__ void sincos_f32(float x, float &s, float &c) {
-    if (fabsf(x) > 8192.0f) {
-        s = sinf(x); c = cosf(x);
-        return;
-    }
     const float k = rintf(x * 0.636619772367581f);
     float r = fmaf(-k, 1.5703125f, x);
     r = fmaf(-k, 4.837512969970703125e-4f, r);
@@ -239,7 +249,11 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
     using frag = typename M::frag;
     constexpr int G = M::G, NP = M::NP;
     constexpr int T1 = kSlots1 / G, T2 = 64 / G;
-    constexpr int NB = NCB == 1 ? 4 : 2;  // row blocks per pass: NB*NCB accumulators of 16 registers
+#ifndef LM_MLPX2_NB
+#define LM_MLPX2_NB 1  // split mode: one accumulator at a time keeps the wave inside 256 registers
+#endif
+    // row blocks per pass: NB*NCB accumulators of 16 registers
+    constexpr int NB = NCB == 1 ? (PREC == LM_MLP_F16X2 ? LM_MLPX2_NB : 4) : 2;
     constexpr int PF = G == 1 ? 4 : 1;
     const unsigned h = lane >> 5;
     frag b2frag[NCB][T2][NP];
@@ -248,18 +262,33 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             float slots[kSlots1];
+            constexpr bool kExact = PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2;
+            bool big = false;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const float x = raw[cb][v];
                 float s1, c1;
-                if (PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2) {
+                if (kExact) {
                     sincos_f32(x, s1, c1);
+                    big |= fabsf(x) > kSincosMax;
                 } else {
                     s1 = __sinf(x); c1 = __cosf(x);
                 }
                 const float s2 = 2.0f * s1 * c1;
                 const float c2 = fmaf(-2.0f * s1, s1, 1.0f);
                 slots[v] = x; slots[16 + v] = s1; slots[32 + v] = c1; slots[48 + v] = s2; slots[64 + v] = c2;
+            }
+            if (kExact && __builtin_expect(big, 0)) {
+                // arguments beyond the fast reduction's range: library routines, rarely if ever taken
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const float x = raw[cb][v];
+                    if (fabsf(x) > kSincosMax) {
+                        const float s1 = sinf(x), c1 = cosf(x);
+                        slots[16 + v] = s1; slots[32 + v] = c1;
+                        slots[48 + v] = 2.0f * s1 * c1; slots[64 + v] = fmaf(-2.0f * s1, s1, 1.0f);
+                    }
+                }
             }
 #pragma unroll
             for (int t = 0; t < T1; ++t) M::pack(slots + t * G, bfrag[cb][t]);
@@ -378,16 +407,24 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
             raw[cb][15] = 0.0f;
         }
     };
+#ifndef LM_MLPX2_PREFETCH
+#define LM_MLPX2_PREFETCH 0  // split mode: the second wave of the SIMD hides the load, the 16 registers are worth more
+#endif
+    // the next tile's inputs travel while this tile is multiplied
+    constexpr bool kPrefetch = PREC != LM_MLP_F16X2 || LM_MLPX2_PREFETCH;
     float nxt[NCB][16];
-    if (wave_id < n_tiles) fetch(wave_id, nxt);
+    if (kPrefetch && wave_id < n_tiles) fetch(wave_id, nxt);
     for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
         float raw[NCB][16];
+        if (kPrefetch) {
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb)
+            for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) raw[cb][v] = nxt[cb][v];
-        // the next tile's inputs travel while this tile is multiplied
-        if (tile + n_waves < n_tiles) fetch(tile + n_waves, nxt);
+                for (int v = 0; v < 16; ++v) raw[cb][v] = nxt[cb][v];
+            if (tile + n_waves < n_tiles) fetch(tile + n_waves, nxt);
+        } else {
+            fetch(tile, raw);
+        }
         float out[NCB][3];
         colour_network<PREC, NCB>(w1, w2, w3, b1, b2, b3, raw, lane, out);
 #pragma unroll

@@ -206,6 +206,28 @@ def test_colour_network(gpu_lib, prec, tol):
         assert (got - ref).abs().max().item() < tol, (M, prec)
 
 
+@pytest.mark.parametrize("prec", ["f32", "f16x2"])
+def test_colour_network_large_arguments(gpu_lib, prec):
+    """Features far outside the fast sine / cosine reduction's range (|x| > 8192) take the library routines: the
+    encoding stays float-accurate.  Weights are scaled down so that the raw features do not saturate the network.
+    The split-fp16 mode carries features as two halves, so its inputs must stay below the fp16 maximum (65504)."""
+    p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48)
+    # the columns of the raw features and view direction: scaled down, or switched off where such small weights
+    # would be fp16 subnormals; the large arguments then act through the sine / cosine columns alone
+    p.mlp_w[0][:, :30] *= 1e-5 if prec == "f32" else 0.0
+    g = torch.Generator().manual_seed(8)
+    feats, view = torch.randn(257, 27, generator=g), torch.randn(257, 3, generator=g)
+    if prec == "f32":
+        feats[::3] *= 3.0e4
+        feats[1::7] *= 2.0e6
+    else:
+        feats[::3] = (feats[::3] * 1.5e4).clamp(-6.0e4, 6.0e4)
+    view[::5] *= 1.0e4
+    got = _model(p).render_module(view, feats, precision=prec).cpu()
+    ref = O.mlp_render(p, view, feats)
+    assert (got - ref).abs().max().item() < 2e-5
+
+
 @pytest.mark.parametrize("prec,tol", [("f32", 2e-6), ("f16x2", 3e-6), ("f16", 2e-3)])
 def test_basis_projection(gpu_lib, prec, tol):
     p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48, ndims=3, resMode=(1, 2))
