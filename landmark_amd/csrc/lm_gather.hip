@@ -620,46 +620,57 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
         int t = 0;  // running MFMA step over the concatenated channels
         // Both samples' footprints of a plane are loaded with every load issued before the first use
         // (one memory round trip per plane), and the loads of plane k + 1 are issued before the
-        // matrix step of plane k, which then runs under their latency.
+        // matrix step of plane k, which then runs under their latency.  Where that many loads in
+        // flight would not fit the registers (wide planes), one sample's loads at a time.
+        constexpr bool kAhead = 2 * NG * 6 * V <= 144;
         Taps2 t2[2];
         Taps1 t1[2];
         Footprint<T> fp[2][NG];
-        auto issue = [&](int k) {
+        auto taps_pass = [&](int k, int pass) {
+            const lm_plane &pl = ps.p[k];
+            const float *q = pass ? q1 : q0;
+            t2[pass] = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
+            t1[pass] = line_taps(pl, pick(q, pl.axl));
+            block_taps(pl, ps.nblk, q, t2[pass], t1[pass]);
+        };
+        auto load_pass = [&](int k, int pass) {
             const lm_plane &pl = ps.p[k];
 #pragma unroll
-            for (int pass = 0; pass < 2; ++pass) {
-                const float *q = pass ? q1 : q0;
-                t2[pass] = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
-                t1[pass] = line_taps(pl, pick(q, pl.axl));
-                block_taps(pl, ps.nblk, q, t2[pass], t1[pass]);
+            for (int gi = 0; gi < NG; ++gi) {
+                const int c = V * (int)qlane + gi * V * kQuad;
+                if (c < C) footprint_load<T>(pl, t2[pass], t1[pass], c, fp[pass][gi]);
             }
-#pragma unroll
-            for (int pass = 0; pass < 2; ++pass)
-#pragma unroll
-                for (int gi = 0; gi < NG; ++gi) {
-                    const int c = V * (int)qlane + gi * V * kQuad;
-                    if (c < C) footprint_load<T>(pl, t2[pass], t1[pass], c, fp[pass][gi]);
-                }
         };
-        issue(0);
+        auto emit_pass = [&](int pass) {
+            float *row = tile + (pass * 16 + gs) * ROW;
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) {
+                const int c = V * (int)qlane + gi * V * kQuad;
+                if (c >= C) continue;
+                float prod[V];
+                footprint_products<T>(fp[pass][gi], t2[pass], t1[pass], prod);
+#pragma unroll
+                for (int i = 0; i < V; i += 4)
+                    *reinterpret_cast<float4 *>(row + c + i) = make_float4(prod[i], prod[i + 1], prod[i + 2], prod[i + 3]);
+            }
+        };
+        if (kAhead) { taps_pass(0, 0); taps_pass(0, 1); load_pass(0, 0); load_pass(0, 1); }
         for (int k = 0; k < ps.n; ++k) {
-            __builtin_amdgcn_sched_barrier(0);
+            if (kAhead) {
+                __builtin_amdgcn_sched_barrier(0);
+                emit_pass(0);
+                emit_pass(1);
+                __builtin_amdgcn_sched_barrier(0);
+                if (k + 1 < ps.n) { taps_pass(k + 1, 0); taps_pass(k + 1, 1); load_pass(k + 1, 0); load_pass(k + 1, 1); }
+            } else {
 #pragma unroll
-            for (int pass = 0; pass < 2; ++pass) {
-                float *row = tile + (pass * 16 + gs) * ROW;
-#pragma unroll
-                for (int gi = 0; gi < NG; ++gi) {
-                    const int c = V * (int)qlane + gi * V * kQuad;
-                    if (c >= C) continue;
-                    float prod[V];
-                    footprint_products<T>(fp[pass][gi], t2[pass], t1[pass], prod);
-#pragma unroll
-                    for (int i = 0; i < V; i += 4)
-                        *reinterpret_cast<float4 *>(row + c + i) = make_float4(prod[i], prod[i + 1], prod[i + 2], prod[i + 3]);
+                for (int pass = 0; pass < 2; ++pass) {
+                    taps_pass(k, pass);
+                    load_pass(k, pass);
+                    __builtin_amdgcn_sched_barrier(0);
+                    emit_pass(pass);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
-            if (k + 1 < ps.n) issue(k + 1);
             __builtin_amdgcn_sched_barrier(0);
             // LDS operations of one wave complete in order; the fence only pins the compiler
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
