@@ -36,8 +36,8 @@ MLP_FLOP_PER_ROW = 2 * (150 * 128 + 128 * 128 + 128 * 3)
 # by the factors a plain copy of known size gave: 2.00 and 1.00) of the default workload's gather
 # kernels at the default chunk size; any other configuration reports null.
 MEASURED_TRAFFIC = {
-    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_app_feat"): 17.15e9 + 0.41e9,
-    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_march"): 9.80e9 + 0.15e9,
+    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_app_feat"): 17.35e9 + 0.42e9,
+    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_march"): 9.77e9 + 0.15e9,
 }
 
 
@@ -74,7 +74,10 @@ def bench_frame(args, workload):
         name = f"c5_4k_cityblock_res{args.base * 8}"
     else:
         raise ValueError(workload)
-    term_eps = 1e-4 / float(p.near_far[1]) if args.term_eps == "auto" else float(args.term_eps)
+    if args.mlp == "auto":
+        args.mlp = "f16" if p.app_plane[0].dtype == torch.float16 else "f16x2"
+    term_auto = args.term_eps == "auto"
+    term_eps = 1e-4 / float(p.near_far[1]) if term_auto else float(args.term_eps)
     args.term_eps = term_eps
     model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=term_eps)
     torch.cuda.synchronize()
@@ -157,7 +160,10 @@ def bench_frame(args, workload):
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
     roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
     roof["launches_per_frame"] = launches
-    roof["traffic"] = MEASURED_TRAFFIC.get((name, chunk, roof["kernel"]))
+    if roof["kernel"] == "k_app_feat" and args.mlp == "f32":
+        roof["kernel"] = "k_app_list+k_basis"  # fp32 matrix mode: products through memory, then basis_mat
+    measured = term_auto and args.mlp == "f16x2" and int(model.ray_row_length) == W
+    roof["traffic"] = MEASURED_TRAFFIC.get((name, chunk, roof["kernel"])) if measured else None
     if roof["traffic"]:
         # the same launch priced by its counter-derived L2-miss traffic instead of the gather-convention bytes
         roof["traffic_GBps"] = round(roof["traffic"] / (roof["avg_launch_ms"] * 1e-3) / 1e9, 1)
@@ -167,7 +173,7 @@ def bench_frame(args, workload):
     out = {
         "metric": "render_throughput", "value": round(mrays, 3), "unit": "Mrays/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32" if args.mlp == "f32" else f"f32+{args.mlp}-mlp",
+        "scaling": "weak", "vs_baseline": None, "dtype": ("f16" if p.app_plane[0].dtype == torch.float16 else "f32") + ("" if args.mlp == "f32" else f"+{args.mlp}-mlp"),
         "data": "synthetic",
         "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "ray_row_hint": int(model.ray_row_length), "mlp": args.mlp,
                    "term_eps": args.term_eps, "valid_samples": n_valid, "marched_samples": n_marched, "app_samples": n_app},
@@ -266,7 +272,7 @@ def bench_mlp(args):
 
     dev = "cuda:0"
     p = scenes.make_params(seed=3, gridSize=(8, 8, 8), density_n_comp=4, app_n_comp=48)
-    prec = args.mlp
+    prec = args.mlp = "f16" if args.mlp == "auto" else args.mlp  # the isolated network is quoted with fp16 weights
     model = GridNeRFHIP(p, device=dev, mlp_precision=prec)
     M = args.rows
     g = torch.Generator(device=dev).manual_seed(3)
@@ -320,7 +326,9 @@ def main():
     ap.add_argument("--width", type=int, default=1920)
     ap.add_argument("--frame", type=int, default=0)
     ap.add_argument("--density-shift", type=float, default=0.0)
-    ap.add_argument("--mlp", default="f16x2", choices=["f32", "f16x2", "f16", "bf16"])
+    ap.add_argument("--mlp", default="auto", choices=["auto", "f32", "f16x2", "f16", "bf16"],
+                    help="arithmetic of the colour network; auto = f16x2 (1e-4 class) with fp32 tables, f16 (1e-2 class) "
+                         "where the tables are fp16 already")
     ap.add_argument("--term-eps", default="auto",
                     help="ray termination threshold on the transmittance; 'auto' = 1e-4 / far, the largest value that "
                          "keeps rgb and depth within 1e-4 of the unterminated render; 0 = never terminate")
