@@ -158,6 +158,9 @@ def bench_frame(args, workload):
         ach = stages[dom]["GBps"]
         roof = {"kernel": "k_march" if dom == "density_march" else "k_app_feat", "bound": "hbm", "achieved": ach,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
+    if roof["bound"] == "hbm":
+        roof["note"] = ("achieved = gather-convention bytes (every corner load of every sample, no reuse between samples) "
+                        "per launch / launch time; traffic = counter-derived HBM-side bytes of the same launch")
     roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
     roof["launches_per_frame"] = launches
     if roof["kernel"] == "k_app_feat" and args.mlp == "f32":
