@@ -120,6 +120,32 @@ def bench_frame(args, workload):
     dt = time.perf_counter() - t0
     ms_step = dt / args.steps * 1e3
 
+    # the same frames when the boundary hands over host buffers: rays from pinned host memory, rgb and depth back to
+    # it, copies and kernels on the one stream (reported beside the metric, never as the metric)
+    ms_host_io = None
+    if args.host_io:
+        rays_h = torch.empty(rays.shape, dtype=rays.dtype, pin_memory=True).copy_(rays)
+        rgb_h = torch.empty(rgb.shape, dtype=rgb.dtype, pin_memory=True)
+        depth_h = torch.empty(depth.shape, dtype=depth.dtype, pin_memory=True)
+        rays_d = torch.empty_like(rays)
+
+        def frame_io():
+            for ci in range(n_chunks):
+                sl = slice(ci * chunk, min((ci + 1) * chunk, N))
+                rays_d[sl].copy_(rays_h[sl], non_blocking=True)
+                model.render_into(rays_d[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci])
+                rgb_h[sl].copy_(rgb[sl], non_blocking=True)
+                depth_h[sl].copy_(depth[sl], non_blocking=True)
+
+        frame_io()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            frame_io()
+        torch.cuda.synchronize()
+        ms_host_io = (time.perf_counter() - t0) / args.steps * 1e3
+        assert torch.equal(rgb_h, rgb.cpu())
+
     cnt = counters.cpu().long() & 0xFFFFFFFF
     n_valid, n_app = int(cnt[:, L.LM_STAT_N_VALID].sum()), int(cnt[:, L.LM_STAT_N_APP].sum())
     n_marched = int(cnt[:, L.LM_STAT_N_MARCHED].sum())
@@ -185,6 +211,8 @@ def bench_frame(args, workload):
         "gather_frac_of_hbm_peak": round(stages["density_march"]["GBps"] / HBM_PEAK_GBS, 4),
         "stages": stages, "roofline": roof, "cpu_baseline": cpu, "parity": parity,
     }
+    if ms_host_io is not None:
+        out["ms_per_step_host_buffers"] = round(ms_host_io, 4)
     return out
 
 
@@ -342,6 +370,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=270)
     ap.add_argument("--cpu-threads", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--host-io", action="store_true", help="also time the frame with rays and results in pinned host memory")
     ap.add_argument("--no-row-hint", action="store_true", help="do not tell the library that rays are image rows")
     ap.add_argument("--calib", action="store_true", help="also run one 1 GiB device copy (counter calibration)")
     args = ap.parse_args()

@@ -154,11 +154,15 @@ int check_model(const lm_model *m, int *K) {
     int dt;
     if (int rc = lm_check_planes(m->density, m->n_planes, &dt, nullptr)) return rc;
     if (int rc = lm_check_planes(m->app, m->n_planes, &dt, K)) return rc;
-    if (m->geom.div0 > 0)
-        for (int k = 0; k < m->n_planes; ++k)
-            for (const lm_plane *pl : {&m->density[k], &m->app[k]})
+    const int64_t blocks = m->geom.div0 > 0 ? (int64_t)m->geom.div0 * m->geom.div1 : 1;
+    for (int k = 0; k < m->n_planes; ++k)
+        for (const lm_plane *pl : {&m->density[k], &m->app[k]}) {
+            // line tables are addressed with 32-bit element offsets
+            LM_REQUIRE((int64_t)pl->Len * pl->C * blocks < ((int64_t)1 << 31), "plane %d: line table too large", k);
+            if (m->geom.div0 > 0)
                 LM_REQUIRE(pl->ax0 == 0 && pl->ax1 == 1 && pl->axl == 2,
                            "a block-stacked model has XY planes and z lines only (plane %d)", k);
+        }
     return LM_OK;
 }
 }  // namespace
