@@ -31,6 +31,7 @@ struct PlaneSet {
 
 template <typename T> struct Vec;
 template <> struct Vec<float> {
+    using elem = float;
     static constexpr int V = 4;
     __device__ static __forceinline__ void load(const float *p, float *o) {
         float4 v = *reinterpret_cast<const float4 *>(p);
@@ -38,6 +39,7 @@ template <> struct Vec<float> {
     }
 };
 template <> struct Vec<__half> {
+    using elem = __half;
     static constexpr int V = 8;
     __device__ static __forceinline__ void load(const __half *p, float *o) {
         uint4 raw = *reinterpret_cast<const uint4 *>(p);
@@ -47,6 +49,19 @@ template <> struct Vec<__half> {
             float2 f = __half22float2(h[i]);
             o[2 * i] = f.x; o[2 * i + 1] = f.y;
         }
+    }
+};
+// fp16 tables read four channels (8 bytes) per lane: for 16- and 48-channel planes, where
+// 16-byte loads would leave half of a quad idle on the last 16 channels
+struct Half4 {};
+template <> struct Vec<Half4> {
+    using elem = __half;
+    static constexpr int V = 4;
+    __device__ static __forceinline__ void load(const __half *p, float *o) {
+        const uint2 raw = *reinterpret_cast<const uint2 *>(p);
+        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+        const float2 a = __half22float2(h[0]), b = __half22float2(h[1]);
+        o[0] = a.x; o[1] = a.y; o[2] = b.x; o[3] = b.y;
     }
 };
 
@@ -118,8 +133,9 @@ __device__ __forceinline__ float pick(const float *q, int ax) { return ax == 0 ?
 template <typename T>
 __device__ __forceinline__ void plane_products(const lm_plane &pl, const Taps2 &t2, const Taps1 &t1, int c, float *prod) {
     constexpr int V = Vec<T>::V;
-    const T *P = reinterpret_cast<const T *>(pl.plane);
-    const T *Ln = reinterpret_cast<const T *>(pl.line);
+    using E = typename Vec<T>::elem;
+    const E *P = reinterpret_cast<const E *>(pl.plane);
+    const E *Ln = reinterpret_cast<const E *>(pl.line);
     float a[V], b[V], cc[V], d[V], l0[V], l1[V];
     Vec<T>::load(P + t2.o00 + c, a);
     Vec<T>::load(P + t2.o01 + c, b);
@@ -176,8 +192,9 @@ template <typename T> struct Footprint {
 };
 template <typename T>
 __device__ __forceinline__ void footprint_load(const lm_plane &pl, const Taps2 &t2, const Taps1 &t1, int c, Footprint<T> &f) {
-    const T *P = reinterpret_cast<const T *>(pl.plane);
-    const T *Ln = reinterpret_cast<const T *>(pl.line);
+    using E = typename Vec<T>::elem;
+    const E *P = reinterpret_cast<const E *>(pl.plane);
+    const E *Ln = reinterpret_cast<const E *>(pl.line);
     Vec<T>::load(P + t2.o00 + c, f.a);
     Vec<T>::load(P + t2.o01 + c, f.b);
     Vec<T>::load(P + t2.o10 + c, f.c);
@@ -198,50 +215,55 @@ __device__ __forceinline__ void footprint_products(const Footprint<T> &f, const 
     }
 }
 
-// Two samples at once (the marching kernel's look-ahead): the loads of both are issued before
-// either is used, so a ray's chain of dependent memory round trips is half as long.  Same
+// NS samples at once (the marching kernel's look-ahead): the loads of all are issued before any
+// is used, so a ray's chain of dependent memory round trips is NS times shorter.  Same
 // operations per sample as density_sum, hence the same bits.
-template <typename T>
-__device__ __forceinline__ void density_sum2(const PlaneSet &ps, const float *qa, const float *qb, unsigned qlane,
-                                             const float *__restrict__ den_w, float &out_a, float &out_b) {
+template <typename T, int NS>
+__device__ __forceinline__ void density_sum_n(const PlaneSet &ps, const float (*q)[4], unsigned qlane,
+                                              const float *__restrict__ den_w, float *out) {
     constexpr int V = Vec<T>::V;
-    float sa = 0.0f, sb = 0.0f;
+    float sum[NS];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) sum[n] = 0.0f;
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
         const lm_plane &pl = ps.p[k];
-        Taps2 a2 = plane_taps(pl, pick(qa, pl.ax0), pick(qa, pl.ax1));
-        Taps1 a1 = line_taps(pl, pick(qa, pl.axl));
-        block_taps(pl, ps.nblk, qa, a2, a1);
-        Taps2 b2 = plane_taps(pl, pick(qb, pl.ax0), pick(qb, pl.ax1));
-        Taps1 b1 = line_taps(pl, pick(qb, pl.axl));
-        block_taps(pl, ps.nblk, qb, b2, b1);
+        Taps2 t2[NS];
+        Taps1 t1[NS];
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+            t2[n] = plane_taps(pl, pick(q[n], pl.ax0), pick(q[n], pl.ax1));
+            t1[n] = line_taps(pl, pick(q[n], pl.axl));
+            block_taps(pl, ps.nblk, q[n], t2[n], t1[n]);
+        }
         for (int c = V * qlane; c < pl.C; c += V * kQuad) {
-            Footprint<T> fa, fb;
-            footprint_load<T>(pl, a2, a1, c, fa);
-            footprint_load<T>(pl, b2, b1, c, fb);
-            // keep the twelve loads ahead of the first use
+            Footprint<T> f[NS];
+#pragma unroll
+            for (int n = 0; n < NS; ++n) footprint_load<T>(pl, t2[n], t1[n], c, f[n]);
+            // keep the 6 * NS loads ahead of the first use
             __builtin_amdgcn_sched_barrier(0);
-            float pa[V], pb[V];
-            footprint_products<T>(fa, a2, a1, pa);
-            footprint_products<T>(fb, b2, b1, pb);
-            if (den_w) {
 #pragma unroll
-                for (int i = 0; i < V; ++i) sa = fmaf(den_w[col + c + i], pa[i], sa);
+            for (int n = 0; n < NS; ++n) {
+                float prod[V];
+                footprint_products<T>(f[n], t2[n], t1[n], prod);
+                if (den_w) {
 #pragma unroll
-                for (int i = 0; i < V; ++i) sb = fmaf(den_w[col + c + i], pb[i], sb);
-            } else {
+                    for (int i = 0; i < V; ++i) sum[n] = fmaf(den_w[col + c + i], prod[i], sum[n]);
+                } else {
 #pragma unroll
-                for (int i = 0; i < V; ++i) sa += pa[i];
-#pragma unroll
-                for (int i = 0; i < V; ++i) sb += pb[i];
+                    for (int i = 0; i < V; ++i) sum[n] += prod[i];
+                }
             }
         }
         col += pl.C;
     }
-    sa += __shfl_xor(sa, 1); sb += __shfl_xor(sb, 1);
-    sa += __shfl_xor(sa, 2); sb += __shfl_xor(sb, 2);
-    out_a = den_w ? fmaxf(sa, 0.0f) : sa;
-    out_b = den_w ? fmaxf(sb, 0.0f) : sb;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+        float v = sum[n];
+        v += __shfl_xor(v, 1);
+        v += __shfl_xor(v, 2);
+        out[n] = den_w ? fmaxf(v, 0.0f) : v;
+    }
 }
 
 // Same sum with a compile-time channel count shared by all planes: the channel groups of a
@@ -435,7 +457,7 @@ __global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int
 // before the density of the samples behind is ever fetched.  With term_eps = 0 the weights
 // are those of the separate density + weights kernels, bit for bit (same operations, and the
 // transmittance is the same sequential product torch.cumprod forms, app/tools/utils.py:51-64).
-template <typename T>
+template <typename T, int NS>  // NS samples of a ray per round
 __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
                                                   const float *__restrict__ rays, const uint64_t *__restrict__ bitmap,
                                                   const uint32_t *__restrict__ p_first,
@@ -490,29 +512,35 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
         }
         if (!__any(have)) break;
         if (have) {
-            // up to two samples per round: both densities are gathered together, the weights follow in order
-            uint64_t flat_a, flat_b = 0;
-            bool finish = !it.next(flat_a);
-            if (!finish) {
-                const bool two = it.next(flat_b);
-                const int s_a = (int)(flat_a - flat0), s_b = two ? (int)(flat_b - flat0) : s_a;
-                const float z_a = lm_sample_z(g, rp, s_a), z_b = lm_sample_z(g, rp, s_b);
-                float pt[3], q_a[4], q_b[4];
-                lm_point(ray, z_a, pt);
-                lm_normalise(g, pt, q_a);
-                q_a[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q_a) : 0);
-                lm_point(ray, z_b, pt);
-                lm_normalise(g, pt, q_b);
-                q_b[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q_b) : 0);
-                float f_a, f_b;
-                density_sum2<T>(ps, q_a, q_b, qlane, den_w, f_a, f_b);
-                marched += two ? 2u : 1u;
+            // up to NS samples per round: their densities are gathered together, the weights follow in order
+            uint64_t flat[NS];
+            int n_have = 0;
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    if (h == 1 && (!two || finish)) break;
-                    const int s = h ? s_b : s_a;
-                    const float z = h ? z_b : z_a;
-                    const float sig = activate(h ? f_b : f_a, act, shift);
+            for (int n = 0; n < NS; ++n) {
+                flat[n] = n ? flat[n - 1] : 0;
+                if (n_have == n && it.next(flat[n])) n_have = n + 1;
+            }
+            bool finish = n_have == 0;
+            if (!finish) {
+                int s_n[NS];
+                float z_n[NS], q[NS][4], f[NS];
+#pragma unroll
+                for (int n = 0; n < NS; ++n) {
+                    s_n[n] = (int)(flat[n < n_have ? n : 0] - flat0);  // missing samples repeat the first (result unused)
+                    z_n[n] = lm_sample_z(g, rp, s_n[n]);
+                    float pt[3];
+                    lm_point(ray, z_n[n], pt);
+                    lm_normalise(g, pt, q[n]);
+                    q[n][3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q[n]) : 0);
+                }
+                density_sum_n<T, NS>(ps, q, qlane, den_w, f);
+                marched += (uint32_t)n_have;
+#pragma unroll
+                for (int n = 0; n < NS; ++n) {
+                    if (n >= n_have || finish) break;
+                    const int s = s_n[n];
+                    const float z = z_n[n];
+                    const float sig = activate(f[n], act, shift);
                     const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
                     const float d2 = dist * distance_scale;
                     const float alpha = 1.0f - expf(-sig * d2);
@@ -525,7 +553,7 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                     ++p;
                     finish = term_eps > 0.0f && Tr < term_eps;
                 }
-                if (!two) finish = true;  // the ray's last sample
+                if (n_have < NS) finish = true;  // the ray's last samples
             }
             if (finish) {
                 if (qlane == 0) {
@@ -547,28 +575,6 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
 // plane by line and feeds the products straight into the matrix cores as the B operand of
 // basis_mat (A = the packed basis fragments, resident in LDS).  The [n, P*L*C] product
 // matrix never exists in memory; the kernel writes the 27 projected features per sample.
-template <typename T, int CW> struct ChLoad;
-template <int CW> struct ChLoad<float, CW> {
-    __device__ static __forceinline__ void load(const float *p, float *o) {
-#pragma unroll
-        for (int i = 0; i < CW; i += 4) {
-            float4 v = *reinterpret_cast<const float4 *>(p + i);
-            o[i] = v.x; o[i + 1] = v.y; o[i + 2] = v.z; o[i + 3] = v.w;
-        }
-    }
-};
-template <> struct ChLoad<__half, 8> {
-    __device__ static __forceinline__ void load(const __half *p, float *o) { Vec<__half>::load(p, o); }
-};
-template <> struct ChLoad<__half, 4> {
-    __device__ static __forceinline__ void load(const __half *p, float *o) {
-        uint2 raw = *reinterpret_cast<const uint2 *>(p);
-        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
-        float2 a = __half22float2(h[0]), b = __half22float2(h[1]);
-        o[0] = a.x; o[1] = a.y; o[2] = b.x; o[3] = b.y;
-    }
-};
-
 template <int PREC> struct AppFeatBlock { static constexpr int N = 512; };
 
 // LDS: [basis fragments | one product tile per wave].  A tile is 32 samples x (C + 4) floats.
@@ -915,6 +921,7 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
     const uint32_t *cnt = counters + LM_STAT_N_APP;
 #define LM_AF_GO(PREC_)                                                                                    \
     return dtype == LM_F32 ? launch_app_feat<PREC_, float>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
+           : (nu & 1)      ? launch_app_feat<PREC_, Half4>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
                            : launch_app_feat<PREC_, __half>(nu, m, ps, K, rays, app_idx, cnt, feat, st)
     switch (m->mlp_prec) {
         case LM_MLP_F16: LM_AF_GO(LM_MLP_F16);
@@ -934,14 +941,23 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
     const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
     const unsigned grid = (unsigned)lm_persistent_blocks(4);
-    if (dtype == LM_F32)
-        hipLaunchKernelGGL(k_march<float>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
-                           p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,
-                           m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
-    else
-        hipLaunchKernelGGL(k_march<__half>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,
-                           p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,
-                           m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched);
+    int c_max = 0;
+    for (int k = 0; k < m->n_planes; ++k) c_max = std::max(c_max, (int)m->density[k].C);
+#define LM_MARCH(T_, NS_)                                                                                              \
+    hipLaunchKernelGGL((k_march<T_, NS_>), dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,   \
+                       p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,            \
+                       m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched)
+    // few narrow fp16 planes: a round is short and light on registers, four samples per round keep more loads
+    // in flight (16.6 -> 14.3 ms on three 8192 x 8192 x 16 planes; with fp32 planes the registers cost more)
+    const bool deep = m->n_planes <= 4;
+    if (dtype == LM_F32) {
+        LM_MARCH(float, 2);
+    } else if (c_max <= 16) {  // 16-byte loads would leave half of every quad idle
+        if (deep) LM_MARCH(Half4, 4); else LM_MARCH(Half4, 2);
+    } else {
+        LM_MARCH(__half, 2);
+    }
+#undef LM_MARCH
     LM_CHECK_LAUNCH("k_march");
     return LM_OK;
 }

@@ -404,11 +404,17 @@ def test_row_length_hint_changes_nothing(gpu_lib, S, width):
     assert a["rgb_map"].min() < 0.99
 
 
-def test_early_termination_bounds(gpu_lib):
-    p = _scene(S=128)
+@pytest.mark.parametrize("fp16_tables,res", [(False, (1,)), (True, (1,)), (True, (1, 2))])
+def test_early_termination_bounds(gpu_lib, fp16_tables, res):
+    """fp32 planes march two samples per round, three narrow fp16 planes four, six of them two."""
+    p = _scene(S=128, resMode=res)
+    if fp16_tables:
+        p = O.to_fp16_features(p)
     rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
     exact, _ = _model(p)(rays)
     term, _ = _model(p, term_eps=1e-4)(rays)
+    ref = O.render_chunk(p, rays)
+    assert (exact["rgb_map"].cpu() - ref["rgb_map"]).abs().max().item() <= (RGB_TOL_16 if fp16_tables else RGB_TOL_F32)
     # all samples after T < 1e-4 have weight < 1e-4 < threshold: colour unchanged up to the white
     # background term (<= 1e-4); depth loses at most T * z_far
     assert (term["rgb_map"] - exact["rgb_map"]).abs().max().item() <= 1e-4
