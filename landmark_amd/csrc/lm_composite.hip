@@ -112,10 +112,20 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
     const uint64_t r = lm_ray_order((uint32_t)o, (uint32_t)N, row);
     float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f;
     const uint32_t first = app_first[r], n = app_cnt[r];
-    for (uint32_t i = 0; i < n; ++i) {
-        const float w = app_w[first + i];
-        const float *c = rgb + 3 * (size_t)(first + i);
-        c0 = fmaf(w, c[0], c0); c1 = fmaf(w, c[1], c1); c2 = fmaf(w, c[2], c2);
+    // four slots per trip, all sixteen loads issued before the sums (which stay in slot order)
+    for (uint32_t i = 0; i < n; i += 4) {
+        float w[4], c[4][3];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t s = first + (i + u < n ? i + u : n - 1);
+            w[u] = app_w[s];
+            c[u][0] = rgb[3 * (size_t)s]; c[u][1] = rgb[3 * (size_t)s + 1]; c[u][2] = rgb[3 * (size_t)s + 2];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u < n) {
+                c0 = fmaf(w[u], c[u][0], c0); c1 = fmaf(w[u], c[u][1], c1); c2 = fmaf(w[u], c[u][2], c2);
+            }
     }
     if (white_bg) {
         const float bgd = 1.0f - acc[r];
@@ -184,13 +194,20 @@ __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const u
         it.start_at(bitmap, r * (uint64_t)S, (r + 1) * (uint64_t)S, p_first[r]);
         const uint32_t end = p_end[r];
         uint64_t flat;
-        for (uint32_t p = it.pos; p < end; ++p) {
-            it.next(flat);
-            const float wgt = w_valid[p];
-            if (wgt > weight_thres) {
-                app_idx[slot] = (uint32_t)flat;
-                app_w[slot] = wgt;
-                ++slot;
+        // four weights per trip so that their loads overlap; the walk over the bitmap stays in order
+        for (uint32_t p = it.pos; p < end; p += 4) {
+            float wgt[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) wgt[u] = w_valid[p + u < end ? p + u : end - 1];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (p + u >= end) break;
+                it.next(flat);
+                if (wgt[u] > weight_thres) {
+                    app_idx[slot] = (uint32_t)flat;
+                    app_w[slot] = wgt[u];
+                    ++slot;
+                }
             }
         }
     }
