@@ -189,8 +189,6 @@ def bench_frame(args, workload):
                         "per launch / launch time; traffic = counter-derived HBM-side bytes of the same launch")
     roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
     roof["launches_per_frame"] = launches
-    if roof["kernel"] == "k_app_feat" and args.mlp == "f32":
-        roof["kernel"] = "k_app_list+k_basis"  # fp32 matrix mode: products through memory, then basis_mat
     measured = term_auto and args.mlp == "f16x2" and int(model.ray_row_length) == W
     roof["traffic"] = MEASURED_TRAFFIC.get((name, chunk, roof["kernel"])) if measured else None
     if roof["traffic"]:

@@ -594,9 +594,9 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
     constexpr int V = Vec<T>::V;
     constexpr int C = 16 * NU, ROW = C + 4;
     constexpr int NG = (C + V * kQuad - 1) / (V * kQuad);  // 16-byte loads per lane, corner and plane
-    static_assert(Mm::G == 8 && Mm::CW == 8, "the fused gather feeds 16-bit MFMAs");
+    constexpr int G = Mm::G, CW = Mm::CW;
     extern __shared__ __align__(16) char lds[];
-    const size_t basis_bytes = (size_t)32 * K * sizeof(typename Mm::elem) * NP;
+    const size_t basis_bytes = (size_t)32 * K * sizeof(typename Mm::elem) * NP;  // K MFMA K-slots x 32 rows
     {
         const uint4 *src = reinterpret_cast<const uint4 *>(packed + L.basis);
         uint4 *dst = reinterpret_cast<uint4 *>(lds);
@@ -682,19 +682,28 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // a lane-half reads CW consecutive channels of every 2*CW and feeds them G at a time
+            // (the order lm_mlp_pack lays the basis fragments out in)
 #pragma unroll
-            for (int u = 0; u < NU; ++u, ++t) {
-                const float4 *src = reinterpret_cast<const float4 *>(tile + j * ROW + 16 * u + 8 * (int)h);
-                const float4 x0 = src[0], x1 = src[1];
-                const float c8[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                frag bf[NP];
-                Mm::pack(c8, bf);
-                const frag a0 = A[(t * NP) * 64 + lane];
-                acc = Mm::mma(a0, bf[0], acc);
-                if constexpr (NP == 2) {
-                    const frag a1 = A[(t * NP + 1) * 64 + lane];
-                    acc = Mm::mma(a1, bf[0], acc);
-                    acc = Mm::mma(a0, bf[1], acc);
+            for (int it = 0; it < C / (2 * CW); ++it) {
+                float cw[CW];
+                const float4 *src = reinterpret_cast<const float4 *>(tile + j * ROW + 2 * CW * it + CW * (int)h);
+#pragma unroll
+                for (int i = 0; i < CW / 4; ++i) {
+                    const float4 x = src[i];
+                    cw[4 * i] = x.x; cw[4 * i + 1] = x.y; cw[4 * i + 2] = x.z; cw[4 * i + 3] = x.w;
+                }
+#pragma unroll
+                for (int u = 0; u < CW / G; ++u, ++t) {
+                    frag bf[NP];
+                    Mm::pack(cw + u * G, bf);
+                    const frag a0 = A[(t * NP) * 64 + lane];
+                    acc = Mm::mma(a0, bf[0], acc);
+                    if constexpr (NP == 2) {
+                        const frag a1 = A[(t * NP + 1) * 64 + lane];
+                        acc = Mm::mma(a1, bf[0], acc);
+                        acc = Mm::mma(a0, bf[1], acc);
+                    }
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -892,7 +901,6 @@ extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint3
 
 // True when the fused gather + basis_mat kernel covers this model's appearance planes.
 int lm_app_feat_supported(const lm_model *m) {
-    if (m->mlp_prec == LM_MLP_F32) return 0;  // fp32 MFMAs take the unfused path
     const int C = m->app[0].C;
     for (int k = 0; k < m->n_planes; ++k)
         if (m->app[k].C != C) return 0;
@@ -914,7 +922,7 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
     LM_REQUIRE(rays && app_idx && counters && feat, "null buffer");
     LM_REQUIRE(m->mlp_packed && lm_aligned16(m->mlp_packed), "packed colour-network weights are null or misaligned");
     if (!lm_app_feat_supported(m))
-        LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs a 16-bit matrix mode and equal channel counts of 16..64 in steps of 16");
+        LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs equal channel counts of 16..64 in steps of 16");
     const PlaneSet ps = make_set(m->app, m->n_planes, &m->geom);
     const int nu = m->app[0].C / 16;
     hipStream_t st = (hipStream_t)stream;
@@ -924,6 +932,7 @@ extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint3
            : (nu & 1)      ? launch_app_feat<PREC_, Half4>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
                            : launch_app_feat<PREC_, __half>(nu, m, ps, K, rays, app_idx, cnt, feat, st)
     switch (m->mlp_prec) {
+        case LM_MLP_F32: LM_AF_GO(LM_MLP_F32);
         case LM_MLP_F16: LM_AF_GO(LM_MLP_F16);
         case LM_MLP_BF16: LM_AF_GO(LM_MLP_BF16);
         default: LM_AF_GO(LM_MLP_F16X2);

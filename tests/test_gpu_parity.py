@@ -271,7 +271,7 @@ def test_weights_against_raw2alpha(gpu_lib):
         assert torch.equal(seg, w["app_mask"][r].nonzero()[:, 0] + r * S)
 
 
-@pytest.mark.parametrize("prec,tol", [("f16x2", 5e-6), ("f16", 5e-3), ("bf16", 4e-2)])
+@pytest.mark.parametrize("prec,tol", [("f32", 5e-6), ("f16x2", 5e-6), ("f16", 5e-3), ("bf16", 4e-2)])
 def test_fused_appearance_features(gpu_lib, prec, tol):
     """gather + basis_mat over the appearance list against the oracle's compute_appfeature"""
     p = _scene(S=64, resMode=(1, 2), thre=0.0)
