@@ -78,6 +78,26 @@ __device__ __forceinline__ uint64_t word_of_ray(const lm_geom &g, const float *_
     const float2 a = rp2[0], b = rp2[1], c = rp2[2];
     ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
     const float rp = lm_ray_param(g, ray);
+    // The word's samples lie between its first and last one (the depth tables are monotone, and so is
+    // o + d * z in z).  If that segment, widened by a margin a hundred times the rounding of the
+    // operations involved, stays on the outer side of one face of the box, every sample fails the box
+    // test and the word is zero without visiting them.  Anything doubtful (NaN included) is visited.
+    {
+        const float za = lm_sample_z(g, rp, (int)j * 64), zb = lm_sample_z(g, rp, (int)j * 64 + 63);
+        const float zlo = fminf(za, zb), zhi = fmaxf(za, zb);
+        // the depth is a sum of two terms bounded by |near| and the ray's parameter (or by the depth itself)
+        const float zm = 1e-5f * (fmaxf(fabsf(zlo), fabsf(zhi)) + fabsf(rp) + fabsf(g.near_));
+        bool outside = false;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const float o = ray[k], d = ray[3 + k];
+            const float e0 = d * (zlo - zm), e1 = d * (zhi + zm), e2 = d * (zlo + zm), e3 = d * (zhi - zm);
+            const float lo = o + fminf(fminf(e0, e1), fminf(e2, e3)), hi = o + fmaxf(fmaxf(e0, e1), fmaxf(e2, e3));
+            const float m = 1e-5f * (fabsf(o) + fmaxf(fabsf(lo), fabsf(hi))) + 1e-30f;
+            outside |= (hi + m < g.aabb[k]) | (lo - m > g.aabb[3 + k]);
+        }
+        if (outside) return 0ull;
+    }
     const bool cells0 = g.vol && g.vol_dtype == LM_CELLS && g.vol_thre == 0.0f;
     uint64_t bits = 0;
 #pragma unroll 4
@@ -148,6 +168,52 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
     uint32_t cnt = 0;
 #pragma unroll
     for (unsigned jj = 0; jj < (unsigned)WPR; ++jj) cnt += s_cnt[ray_local * WPR + jj];
+    uint32_t incl = cnt;
+#pragma unroll
+    for (int d = 1; d < LM_WAVE; d <<= 1) {
+        const uint32_t y = __shfl_up(incl, d);
+        if (lane >= (unsigned)d) incl += y;
+    }
+    const uint32_t total = __shfl(incl, LM_WAVE - 1);
+    uint32_t base = 0;
+    if (total) {
+        if (lane == 0) base = atomicAdd(n_valid, total);
+        base = __shfl(base, 0);
+    }
+    const bool any = cnt != 0;
+    if (r < N) {
+        const uint32_t first = base + incl - cnt;
+        p_first[r] = first;
+        if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
+    }
+    lm_ray_enqueue(any && r < N, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
+}
+
+// The same for long rays (four words): one lane per ray takes its words one after the other, so a
+// word outside the box costs a few instructions and no wave waits at a barrier for a slower one
+// (with one lane per word the workgroup lasts as long as its slowest word).  Rays reach the queue
+// in a less regular order this way, which costs the march a little; with one or two words per ray
+// the kernel above is the better trade.
+template <int WPR>
+__global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, const float *__restrict__ rays, uint32_t N,
+                                                            uint32_t row, uint64_t *__restrict__ bitmap,
+                                                            uint32_t *__restrict__ p_first,
+                                                            uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
+                                                            uint32_t *__restrict__ n_valid, float *__restrict__ acc,
+                                                            float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
+                                                            uint32_t *__restrict__ p_end) {
+    const unsigned lane = lm_lane();
+    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;  // position in the visiting order
+    const uint64_t r = o < N ? lm_ray_order((uint32_t)o, N, row) : o;
+    uint32_t cnt = 0;
+    if (r < N) {
+#pragma unroll
+        for (unsigned j = 0; j < (unsigned)WPR; ++j) {
+            const uint64_t bits = word_of_ray(g, rays, r, j);
+            bitmap[r * WPR + j] = bits;
+            cnt += (uint32_t)__popcll(bits);
+        }
+    }
     uint32_t incl = cnt;
 #pragma unroll
     for (int d = 1; d < LM_WAVE; d <<= 1) {
@@ -415,7 +481,10 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
                        ray_list, bins, n_valid, acc, depth, app_cnt, p_end)
     if (wpr == 1) LM_CULL_SETUP(1);
     else if (wpr == 2) LM_CULL_SETUP(2);
-    else LM_CULL_SETUP(4);
+    else
+        hipLaunchKernelGGL(k_cull_rays_setup_serial<4>, dim3((unsigned)(((uint64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt,
+                           p_end);
 #undef LM_CULL_SETUP
     LM_CHECK_LAUNCH("k_cull_rays_setup");
     return LM_OK;
