@@ -81,6 +81,38 @@ def test_sample_cull_ray_per_lane_kernel(gpu_lib, opt, S, thre, mask, occ):
     assert a["n_valid"] == b["n_valid"] and torch.equal(a["bitmap"], b["bitmap"]) and torch.equal(a["word_prefix"], b["word_prefix"])
 
 
+@pytest.mark.parametrize("opt,S", [(0, 128), (1, 128), (1, 256)])
+def test_cull_rays_along_box_faces(gpu_lib, opt, S):
+    """Rays that run in a face of the box, one float above and below it, and through its edges and corners: whole
+    words of samples sit exactly on the boundary of the box test, where the kernel's segment shortcut must stay
+    on the safe side."""
+    p = _scene(opt=opt, S=S, with_mask=False, step_ratio=0.05)
+    lo, hi = p.aabb[0], p.aabb[1]
+    up = lambda x: torch.nextafter(torch.tensor(x), torch.tensor(10.0)).item()
+    dn = lambda x: torch.nextafter(torch.tensor(x), torch.tensor(-10.0)).item()
+    rays = []
+    for ax in range(3):
+        for face in (lo[ax].item(), hi[ax].item()):
+            for c in (face, up(face), dn(face)):
+                for sgn in (1.0, -1.0):
+                    o = [0.1, -0.2, 1.9]
+                    d = [0.3 * sgn, 0.2, -1.0]
+                    if ax == 2:
+                        o, d = [-1.7, 0.05, c], [1.0, 0.1 * sgn, 0.0]
+                    else:
+                        o[ax], d[ax] = c, 0.0
+                    rays.append(o + d)
+    rays.append([lo[0].item(), lo[1].item(), 1.9, 0.0, 0.0, -1.0])  # down a vertical edge
+    rays.append([-1.8, -1.8, 1.8, 1.0, 1.0, -1.0])  # through two corners
+    rays = torch.tensor(rays, dtype=torch.float32)
+    ref = O.render_chunk(p, rays, N_samples=S, return_aux=True)
+    out = _model(p).sample_cull(rays, N_samples=S, want_z=False)
+    assert ref["ray_valid"].any() and not ref["ray_valid"].all()
+    assert torch.equal(out["ray_valid"].cpu(), ref["ray_valid"])
+    res, _ = _model(p)(rays, N_samples=S)  # the one-launch cull of the whole-chunk render takes the same decisions
+    assert (res["depth_map"].cpu() - ref["depth_map"]).abs().max().item() <= RGB_TOL_F32
+
+
 def test_occupancy_lookup_on_voxel_centres(gpu_lib):
     """Sample points that fall exactly on voxel centres and faces of the occupancy grid (zero upper weights):
     the positive-lookup shortcut must agree with the summed lookup."""
