@@ -36,8 +36,8 @@ MLP_FLOP_PER_ROW = 2 * (150 * 128 + 128 * 128 + 128 * 3)
 # by the factors a plain copy of known size gave: 2.00 and 1.00) of the default workload's gather
 # kernels at the default chunk size; any other configuration reports null.
 MEASURED_TRAFFIC = {
-    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_app_feat"): 17.35e9 + 0.42e9,
-    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_march"): 9.77e9 + 0.15e9,
+    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_app_feat"): 17.36e9 + 0.42e9,
+    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_march"): 9.90e9 + 0.15e9,
 }
 
 
@@ -205,8 +205,11 @@ def bench_frame(args, workload):
         "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "ray_row_hint": int(model.ray_row_length), "mlp": args.mlp,
                    "term_eps": args.term_eps, "valid_samples": n_valid, "marched_samples": n_marched, "app_samples": n_app},
         "frames_per_s": round(1e3 / ms_step, 3), "mpixel_per_s": round(mrays, 3),
-        "gather_GBps": stages["density_march"]["GBps"],
-        "gather_frac_of_hbm_peak": round(stages["density_march"]["GBps"] / HBM_PEAK_GBS, 4),
+        # feature gather: gather-convention bytes per second of both gather kernels, and the dominant one's
+        # counter-derived HBM traffic rate against the HBM peak (null where it was not measured)
+        "gather_algorithmic_GBps": {"density": stages["density_march"]["GBps"], "appearance": stages["app_gather"]["GBps"]},
+        "gather_hbm_GBps": roof.get("traffic_GBps"),
+        "gather_frac_of_hbm_peak": round(roof["traffic_GBps"] / HBM_PEAK_GBS, 4) if roof.get("traffic_GBps") else None,
         "stages": stages, "roofline": roof, "cpu_baseline": cpu, "parity": parity,
     }
     if ms_host_io is not None:
