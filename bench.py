@@ -170,6 +170,7 @@ def bench_frame(args, workload):
     cull_B = (1 if model._vol_dtype == L.LM_CELLS else 32 if model._vol is not None else 0) + 0.125
     stages["cull"].update(bytes_per_sample=cull_B, Gsamples_per_s=round(N * S / (stage_ms[0] * 1e-3) / 1e9, 1),
                           GBps=round((N * S * cull_B + N * 24) / (stage_ms[0] * 1e-3) / 1e9, 1))
+    stages["composite"].update(GBps=round((n_app * 16 + N * 32) / max(stage_ms[5], 1e-9) / 1e6, 1))  # w + rgb per slot; first, count, acc in and rgb out per ray
     stages["app_list"].update(GBps=round((n_marched * 4 + N * S / 8 + n_app * 8 + N * 16) / (stage_ms[2] * 1e-3) / 1e9, 1))
 
     # dominant kernel -> roofline object

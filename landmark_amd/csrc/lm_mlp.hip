@@ -253,7 +253,10 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
 #define LM_MLPX2_NB 1  // split mode: one accumulator at a time keeps the wave inside 256 registers
 #endif
     // row blocks per pass: NB*NCB accumulators of 16 registers
-    constexpr int NB = NCB == 1 ? (PREC == LM_MLP_F16X2 ? LM_MLPX2_NB : 4) : 2;
+#ifndef LM_MLP16_NB1
+#define LM_MLP16_NB1 4
+#endif
+    constexpr int NB = NCB == 1 ? (PREC == LM_MLP_F16X2 ? LM_MLPX2_NB : (PREC == LM_MLP_F32 ? 4 : LM_MLP16_NB1)) : 2;
     constexpr int PF = G == 1 ? 4 : 1;
     const unsigned h = lane >> 5;
     frag b2frag[NCB][T2][NP];
