@@ -232,11 +232,25 @@ template <int PREC>
 __device__ __forceinline__ void relu_to_frags(const floatx16 &acc, typename Mma<PREC>::frag (*out)[Mma<PREC>::NP]) {
     using M = Mma<PREC>;
     constexpr int G = M::G;
-    float hv[16];
+    if constexpr (PREC == LM_MLP_F16) {
+        // round first, then clamp two halves per instruction: rounding is monotone and keeps zero, so
+        // this equals rounding relu(x)
+        float hv[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) hv[v] = relu_f32(acc[v]);
+        for (int v = 0; v < 16; ++v) hv[v] = acc[v];
 #pragma unroll
-    for (int u = 0; u < 16 / G; ++u) M::pack(hv + u * G, out[u]);
+        for (int u = 0; u < 16 / G; ++u) {
+            M::pack(hv + u * G, out[u]);
+            const half8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+            out[u][0] = __builtin_elementwise_max(out[u][0], zero);
+        }
+    } else {
+        float hv[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) hv[v] = relu_f32(acc[v]);
+#pragma unroll
+        for (int u = 0; u < 16 / G; ++u) M::pack(hv + u * G, out[u]);
+    }
 }
 
 // raw[cb][16] (the lane's 16 input rows of each of its NCB samples) -> rgb in out[cb][0..2]
