@@ -468,6 +468,25 @@ def test_ray_generation_and_rgba8(gpu_lib):
     assert torch.equal(postprocess_rgba8(rgb.cuda(), 480, 640).cpu(), O.postprocess_rgba8(rgb, 480, 640))
 
 
+def test_render_frame_from_pose(gpu_lib):
+    """Pose -> RGBA8 image in one call: equals rays from the pose, the chunked render and the byte conversion done
+    step by step with the oracle, up to one grey level where a channel sits on a rounding boundary."""
+    from landmark_amd.render import render_frame
+
+    p = _scene(S=64, thre=0.0)
+    H, W, focal = 72, 96, 90.0
+    pose = torch.cat([scenes.orbit_pose(2.6, 1.9, 3), torch.tensor([[0.0], [0.0], [focal]])], 1)
+    m = _model(p, mlp_precision="f16x2")
+    img, dep = render_frame(m, pose, H, W, chunk=20 * W, depth=True)
+    assert img.shape == (H, W, 4) and img.dtype == torch.uint8 and m.ray_row_length == 0
+    ref = O.render_chunk(p, O.generate_rays(pose, H, W))
+    want = O.postprocess_rgba8(ref["rgb_map"], H, W)
+    diff = (img.cpu().int() - want.int()).abs()
+    assert diff.max().item() <= 1 and (diff > 0).float().mean().item() < 0.01
+    assert (dep.cpu().reshape(-1) - ref["depth_map"]).abs().max().item() <= 2 * RGB_TOL_F32
+    assert want[..., :3].min() < 250  # the scene is visible
+
+
 # ------------------------------------------------------------------------------------ occupancy volume from the model
 ALPHA_TOL = 2e-6  # alpha lies in [0, 1]
 
