@@ -384,7 +384,7 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    copy_rate = None
+    copy_rate = stream_rate = None
     if args.calib:
         a = torch.ones(1 << 28, device="cuda:0")  # 1 GiB read + 1 GiB written by one copy kernel
         b = torch.empty_like(a)
@@ -398,6 +398,16 @@ def main():
         torch.cuda.synchronize()
         copy_rate = 20 * 2 * a.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
         log(f"[bench] device copy, 1 GiB: {copy_rate:.0f} GB/s (read + write)")
+        # a plain streaming kernel (one read, one write per element) as a second yardstick
+        torch.add(a, 1.0, out=b)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(20):
+            torch.add(a, 1.0, out=b)
+        e1.record()
+        torch.cuda.synchronize()
+        stream_rate = 20 * 2 * a.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+        log(f"[bench] elementwise add, 1 GiB in, 1 GiB out: {stream_rate:.0f} GB/s (read + write)")
         del a, b
     if args.workload == "c2":
         out = bench_gather(args)
@@ -407,6 +417,7 @@ def main():
         out = bench_frame(args, args.workload)
     if copy_rate is not None:
         out["hbm_copy_GBps"] = round(copy_rate, 1)
+        out["hbm_stream_GBps"] = round(stream_rate, 1)
     print(json.dumps(out), flush=True)
 
 
