@@ -949,11 +949,17 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     if (int rc = lm_check_planes(m->density, m->n_planes, &dtype, nullptr)) return rc;
     LM_REQUIRE(m->act == LM_ACT_SOFTPLUS || m->act == LM_ACT_RELU, "unknown activation %d", m->act);
     const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
-    const unsigned grid = (unsigned)lm_persistent_blocks(4);
+    // as many workgroups as are resident at once (the kernel's register count decides), at most four per CU
+    auto resident_grid = [](const void *kernel) {
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBlock, 0) != hipSuccess || per_cu < 1) per_cu = 2;
+        return (unsigned)lm_persistent_blocks(std::min(per_cu, 4));
+    };
     int c_max = 0;
     for (int k = 0; k < m->n_planes; ++k) c_max = std::max(c_max, (int)m->density[k].C);
 #define LM_MARCH(T_, NS_)                                                                                              \
-    hipLaunchKernelGGL((k_march<T_, NS_>), dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,   \
+    hipLaunchKernelGGL((k_march<T_, NS_>), dim3(resident_grid(reinterpret_cast<const void *>(&k_march<T_, NS_>))),         \
+                       dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,   \
                        p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,            \
                        m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched)
     // few narrow fp16 planes: a round is short and light on registers, four samples per round keep more loads
