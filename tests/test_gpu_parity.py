@@ -581,6 +581,37 @@ def test_stacked_model_random_scene(gpu_lib, div, res, prec):
     assert int(band.sum()) <= max(2, rays.shape[0] // 500)
 
 
+@pytest.mark.parametrize("div", [(2, 3), (5, 4), (7, 1)])
+def test_block_assignment_is_bit_faithful(gpu_lib, div):
+    """Planes that are constant inside a block and differ between blocks (relu activation, one channel set): the density
+    of a sample then names the block it was assigned to, exactly, for every valid sample including those next to block
+    borders; a second model with planes linear in the block-relative x pins those coordinates to float accuracy."""
+    B = div[0] * div[1]
+    p = scenes.make_params(seed=2, gridSize=(6, 5, 7), near_far=[0.5, 4.5], n_importance=128, sampling_opt=1,
+                           density_shift=0.0, resMode=(1,), ndims=1, plane_division=div, fea2denseAct="relu")
+    ids = torch.arange(1, B + 1, dtype=torch.float32)
+    p.density_plane[0].zero_()
+    p.density_plane[0][0, 0] = ids.view(B, 1, 1).expand(B, 5, 6)
+    p.density_line[0].zero_()
+    p.density_line[0][0, 0] = 1.0
+    rays = scenes.pinhole_rays(64, 64, 50.0, scenes.sphere_pose(2.5, 3))
+    ref = O.render_chunk(p, rays, return_aux=True)
+    m = _model(p)
+    cull = m.sample_cull(rays)
+    assert torch.equal(cull["ray_valid"].cpu(), ref["ray_valid"])
+    sig = m.density_valid(cull).cpu()
+    want = ref["sigma"][ref["ray_valid"]]
+    assert len(set(want.round().tolist())) == B  # every block is hit
+    # the reference interpolates over the block axis with a coordinate that is an integer up to rounding
+    assert (sig - want).abs().max().item() <= 1e-5 * B
+    assert torch.equal(sig.round(), want.round())
+    # block-relative x: plane value = column index inside the block
+    p.density_plane[0][0, 0] = torch.arange(6, dtype=torch.float32).view(1, 1, 6).expand(B, 5, 6)
+    ref = O.render_chunk(p, rays, return_aux=True)
+    sig = _model(p).density_valid(cull).cpu()
+    assert (sig - ref["sigma"][ref["ray_valid"]]).abs().max().item() <= 2e-5
+
+
 def test_stacked_checkpoint_round_trip(gpu_lib, tmp_path):
     from landmark_amd import checkpoint
 
