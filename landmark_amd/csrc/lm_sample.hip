@@ -189,13 +189,13 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
     lm_ray_enqueue(any && r < N, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
 }
 
-// The same for long rays (four words): one lane per ray takes its words one after the other, so a
+// The same for long rays (three words and more): one lane per ray takes its words one after the other, so a
 // word outside the box costs a few instructions and no wave waits at a barrier for a slower one
 // (with one lane per word the workgroup lasts as long as its slowest word).  Rays reach the queue
 // in a less regular order this way, which costs the march a little; with one or two words per ray
 // the kernel above is the better trade.
-template <int WPR>
 __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, const float *__restrict__ rays, uint32_t N,
+                                                                   uint32_t WPR,
                                                             uint32_t row, uint64_t *__restrict__ bitmap,
                                                             uint32_t *__restrict__ p_first,
                                                             uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
@@ -207,8 +207,7 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
     const uint64_t r = o < N ? lm_ray_order((uint32_t)o, N, row) : o;
     uint32_t cnt = 0;
     if (r < N) {
-#pragma unroll
-        for (unsigned j = 0; j < (unsigned)WPR; ++j) {
+        for (unsigned j = 0; j < WPR; ++j) {
             const uint64_t bits = word_of_ray(g, rays, r, j);
             bitmap[r * WPR + j] = bits;
             cnt += (uint32_t)__popcll(bits);
@@ -467,13 +466,13 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
     return LM_OK;
 }
 
-// Cull + per-ray set-up in one launch for the whole-chunk render; returns 1 when the sample count has
-// no such kernel (the caller then takes lm_sample_cull + the list kernel), 0 on success.
+// Cull + per-ray set-up in one launch for the whole-chunk render; returns 1 when the sample count is not
+// a multiple of 64 (the caller then takes lm_sample_cull + the list kernel), 0 on success.
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *bins, uint32_t *n_valid, float *acc, float *depth,
                          uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st) {
     const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
-    if (!(wpr == 1 || wpr == 2 || wpr == 4)) return 1;
+    if (wpr == 0) return 1;
     LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
     const unsigned groups = (unsigned)(((uint64_t)N * wpr + kBlock - 1) / kBlock);
 #define LM_CULL_SETUP(W_)                                                                                             \
@@ -482,9 +481,9 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
     if (wpr == 1) LM_CULL_SETUP(1);
     else if (wpr == 2) LM_CULL_SETUP(2);
     else
-        hipLaunchKernelGGL(k_cull_rays_setup_serial<4>, dim3((unsigned)(((uint64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                           st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt,
-                           p_end);
+        hipLaunchKernelGGL(k_cull_rays_setup_serial, dim3((unsigned)(((uint64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           st, *geom, rays, (uint32_t)N, (uint32_t)wpr, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth,
+                           app_cnt, p_end);
 #undef LM_CULL_SETUP
     LM_CHECK_LAUNCH("k_cull_rays_setup");
     return LM_OK;

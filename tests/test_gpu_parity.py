@@ -356,6 +356,15 @@ def test_render_random_scenes(gpu_lib, opt, act, shift, res, ndims):
     assert ref["app_mask"].any(), "scene must exercise the colour network"
 
 
+@pytest.mark.parametrize("opt,S", [(1, 192), (1, 320), (0, 448), (1, 100)])
+def test_render_other_sample_counts(gpu_lib, opt, S):
+    """Multiples of 64 beyond 128 / 256 take the one-launch cull with one lane per ray; anything else the scan path."""
+    p = _scene(opt=opt, S=S, shift=0.0, step_ratio=0.08, thre=0.0)
+    rays = scenes.pinhole_rays(40, 40, 34.0, scenes.sphere_pose(2.5, 9))
+    ref, _ = _check_render(p, rays, RGB_TOL_F32, S=S)
+    assert ref["app_mask"].any()
+
+
 def test_appearance_embedding_and_density_projection(gpu_lib):
     """encode_app (latent folded into the first layer's bias, switched per call) and
     nonlinear_density against the oracle."""
