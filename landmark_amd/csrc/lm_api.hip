@@ -81,9 +81,6 @@ int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *ap
                         const float *rgb, const float *acc, int white_bg, uint32_t row, float *rgb_map,
                         hipStream_t stream);
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
-int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
-                          uint32_t *ray_list, uint32_t *n_active, float *acc, float *depth, uint32_t *app_cnt,
-                          uint32_t *p_end, uint32_t row, hipStream_t stream);
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
                          uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st);
@@ -99,8 +96,6 @@ int lm_launch_basis(int prec, const void *packed, int K, const float *products, 
 namespace {
 struct Workspace {
     uint64_t *bitmap;
-    uint32_t *word_prefix;
-    void *cull_scratch;
     float *w_valid;
     uint32_t *app_first;
     uint32_t *app_cnt;
@@ -129,8 +124,6 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products)
     // every sample may be valid and (for S below 1/threshold) above the weight threshold
     const uint64_t cap = total;
     w.bitmap = (uint64_t *)take(n_words * 8);
-    w.word_prefix = (uint32_t *)take(n_words * 4);
-    w.cull_scratch = take(lm_sample_cull_scratch_bytes(N, S));
     w.w_valid = (float *)take(total * 4);
     w.app_first = (uint32_t *)take((uint64_t)N * 4);
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
@@ -197,18 +190,9 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     const uint32_t row = m->ray_row % 8 == 0 ? (uint32_t)m->ray_row : 0u;  // tiles of 8 x 8 pixels need whole tiles per row
     mark(0);
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
-    // sample counts of 64, 128 or 256: one launch decides the samples and sets the rays up; otherwise the
-    // stage-level cull (scan + per-word prefix) followed by the list kernel
-    int rc_setup = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
-                                        cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, st);
-    if (rc_setup < 0) return rc_setup;
-    if (rc_setup > 0) {
-        if (int rc = lm_sample_cull(&m->geom, rays, N, w.bitmap, w.word_prefix, nullptr, cnt, nullptr, w.cull_scratch, st))
-            return rc;
-        if (int rc = lm_launch_active_rays(S, N, w.bitmap, w.word_prefix, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
-                                           w.acc, depth_map, w.app_cnt, w.p_end, row, st))
-            return rc;
-    }
+    if (int rc = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
+                                      cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, st))
+        return rc;
     mark(LM_STAGE_CULL);
     if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS, (uint32_t)N, cnt + LM_STAT_QUEUE,
                                  w.w_valid, w.acc, depth_map, w.app_cnt, w.p_end, cnt + LM_STAT_N_MARCHED, st))

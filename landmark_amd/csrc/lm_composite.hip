@@ -136,30 +136,6 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
     rgb_map[3 * r + 2] = fminf(fmaxf(c2, 0.0f), 1.0f);
 }
 
-// Rays that have at least one valid sample, for the marching kernel's queue; the others get
-// their (zero) results here.  p_first[r] = compact position of the ray's first valid sample.
-__global__ __launch_bounds__(kBlock) void k_active_rays(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
-                                                        const uint32_t *__restrict__ word_prefix,
-                                                        uint32_t *__restrict__ p_first,
-                                                        uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
-                                                        float *__restrict__ acc, float *__restrict__ depth,
-                                                        uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end,
-                                                        uint32_t row) {
-    const unsigned lane = lm_lane();
-    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-    const uint64_t r = o < N ? lm_ray_order((uint32_t)o, (uint32_t)N, row) : o;
-    bool any = false;
-    if (r < N) {
-        BitWalk it;
-        it.start(bitmap, word_prefix, r * (uint64_t)S, (r + 1) * (uint64_t)S);
-        p_first[r] = it.pos;
-        uint64_t flat;
-        any = it.next(flat);
-        if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = it.pos; }
-    }
-    lm_ray_enqueue(any, 0, (uint32_t)r, ray_list, (uint32_t)N, bins);  // one list: the counts are not known here
-}
-
 // Appearance list from stored weights: a contiguous slot range per ray (wave prefix + one
 // atomic), filled in sample order from the weights of the ray's samples [first, p_end).
 __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
@@ -253,16 +229,6 @@ int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *ap
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
     hipLaunchKernelGGL(k_zero_counters, dim3(1), dim3(64), 0, stream, counters);
     LM_CHECK_LAUNCH("k_zero_counters");
-    return LM_OK;
-}
-
-int lm_launch_active_rays(int S, int64_t N, const uint64_t *bitmap, const uint32_t *word_prefix, uint32_t *p_first,
-                          uint32_t *ray_list, uint32_t *bins, float *acc, float *depth, uint32_t *app_cnt,
-                          uint32_t *p_end, uint32_t row, hipStream_t stream) {
-    const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(k_active_rays, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, word_prefix, p_first,
-                       ray_list, bins, acc, depth, app_cnt, p_end, row);
-    LM_CHECK_LAUNCH("k_active_rays");
     return LM_OK;
 }
 

@@ -10,6 +10,8 @@
 // (app/models/gridnerf_sequential.py:461-465, 472), so indices match it exactly.
 #include <limits.h>
 
+#include <algorithm>
+
 #include "lm_common.h"
 
 namespace {
@@ -72,18 +74,14 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *
 // same few cache lines (a wave of 64 samples along one ray touches 64 different ones), and the
 // per-ray work (slab test or hull distance) is done once per word instead of once per sample.
 // A workgroup covers 256 consecutive words = 4 of the 64-word groups k_scan_blocks counts.
-__device__ __forceinline__ uint64_t word_of_ray(const lm_geom &g, const float *__restrict__ rays, uint64_t r, unsigned j) {
-    float ray[6];
-    const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
-    const float2 a = rp2[0], b = rp2[1], c = rp2[2];
-    ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
-    const float rp = lm_ray_param(g, ray);
-    // The word's samples lie between its first and last one (the depth tables are monotone, and so is
+// Decisions of samples s0 .. s0 + n - 1 (n <= 64) of one ray, sample s0 + i in bit bit0 + i.
+__device__ __forceinline__ uint64_t segment_bits(const lm_geom &g, const float *ray, float rp, int s0, int n, int bit0) {
+    // The samples lie between the first and the last one (the depth tables are monotone, and so is
     // o + d * z in z).  If that segment, widened by a margin a hundred times the rounding of the
     // operations involved, stays on the outer side of one face of the box, every sample fails the box
-    // test and the word is zero without visiting them.  Anything doubtful (NaN included) is visited.
+    // test and the bits are zero without visiting them.  Anything doubtful (NaN included) is visited.
     {
-        const float za = lm_sample_z(g, rp, (int)j * 64), zb = lm_sample_z(g, rp, (int)j * 64 + 63);
+        const float za = lm_sample_z(g, rp, s0), zb = lm_sample_z(g, rp, s0 + n - 1);
         const float zlo = fminf(za, zb), zhi = fmaxf(za, zb);
         // the depth is a sum of two terms bounded by |near| and the ray's parameter (or by the depth itself)
         const float zm = 1e-5f * (fmaxf(fabsf(zlo), fabsf(zhi)) + fabsf(rp) + fabsf(g.near_));
@@ -101,16 +99,29 @@ __device__ __forceinline__ uint64_t word_of_ray(const lm_geom &g, const float *_
     const bool cells0 = g.vol && g.vol_dtype == LM_CELLS && g.vol_thre == 0.0f;
     uint64_t bits = 0;
 #pragma unroll 4
-    for (int i = 0; i < 64; ++i) {
-        const float z = lm_sample_z(g, rp, (int)j * 64 + i);
+    for (int i = 0; i < n; ++i) {
+        const float z = lm_sample_z(g, rp, s0 + i);
         float pt[3];
         lm_point(ray, z, pt);
         bool ok;
         if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
         else ok = lm_sample_valid(g, pt);
-        bits |= (uint64_t)ok << i;
+        bits |= (uint64_t)ok << (bit0 + i);
     }
     return bits;
+}
+
+__device__ __forceinline__ void load_ray(const float *__restrict__ rays, uint64_t r, float *ray) {
+    const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
+    const float2 a = rp2[0], b = rp2[1], c = rp2[2];
+    ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+}
+
+// word j of ray r when S is a multiple of 64
+__device__ __forceinline__ uint64_t word_of_ray(const lm_geom &g, const float *__restrict__ rays, uint64_t r, unsigned j) {
+    float ray[6];
+    load_ray(rays, r, ray);
+    return segment_bits(g, ray, lm_ray_param(g, ray), (int)j * 64, 64, 0);
 }
 
 template <int WPR>
@@ -195,21 +206,29 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
 // in a less regular order this way, which costs the march a little; with one or two words per ray
 // the kernel above is the better trade.
 __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, const float *__restrict__ rays, uint32_t N,
-                                                                   uint32_t WPR,
-                                                            uint32_t row, uint64_t *__restrict__ bitmap,
-                                                            uint32_t *__restrict__ p_first,
-                                                            uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
-                                                            uint32_t *__restrict__ n_valid, float *__restrict__ acc,
-                                                            float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
-                                                            uint32_t *__restrict__ p_end) {
+                                                                   uint32_t row, uint64_t *__restrict__ bitmap,
+                                                                   uint32_t *__restrict__ p_first,
+                                                                   uint32_t *__restrict__ ray_list,
+                                                                   uint32_t *__restrict__ bins,
+                                                                   uint32_t *__restrict__ n_valid, float *__restrict__ acc,
+                                                                   float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
+                                                                   uint32_t *__restrict__ p_end) {
     const unsigned lane = lm_lane();
     const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;  // position in the visiting order
     const uint64_t r = o < N ? lm_ray_order((uint32_t)o, N, row) : o;
     uint32_t cnt = 0;
     if (r < N) {
-        for (unsigned j = 0; j < WPR; ++j) {
-            const uint64_t bits = word_of_ray(g, rays, r, j);
-            bitmap[r * WPR + j] = bits;
+        float ray[6];
+        load_ray(rays, r, ray);
+        const float rp = lm_ray_param(g, ray);
+        // the ray's samples are bits [flat0, flat1) of the bitmap: whole words are stored, a first or last word
+        // shared with a neighbouring ray is merged into the (zeroed) bitmap
+        const uint64_t flat0 = r * (uint64_t)g.S, flat1 = flat0 + (uint64_t)g.S;
+        for (uint64_t w = flat0 >> 6; w * 64 < flat1; ++w) {
+            const uint64_t lo = w * 64 > flat0 ? w * 64 : flat0, hi = (w + 1) * 64 < flat1 ? (w + 1) * 64 : flat1;
+            const uint64_t bits = segment_bits(g, ray, rp, (int)(lo - flat0), (int)(hi - lo), (int)(lo & 63));
+            if (hi - lo == 64) bitmap[w] = bits;
+            else if (bits) atomicOr(reinterpret_cast<unsigned long long *>(bitmap + w), (unsigned long long)bits);
             cnt += (uint32_t)__popcll(bits);
         }
     }
@@ -232,6 +251,11 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
     }
     lm_ray_enqueue(any && r < N, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
+}
+
+// words of the bitmap that two rays share must start at zero (sample counts that are not multiples of 64)
+__global__ __launch_bounds__(kBlock) void k_zero_words(uint64_t *__restrict__ p, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) p[i] = 0ull;
 }
 
 // exclusive scan of n counts by one workgroup of 1024 threads; total -> *total_out
@@ -466,24 +490,30 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
     return LM_OK;
 }
 
-// Cull + per-ray set-up in one launch for the whole-chunk render; returns 1 when the sample count is not
-// a multiple of 64 (the caller then takes lm_sample_cull + the list kernel), 0 on success.
+// Cull + per-ray set-up for the whole-chunk render: one launch (plus a fill of the bitmap when the sample
+// count is not a multiple of 64).
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *bins, uint32_t *n_valid, float *acc, float *depth,
                          uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st) {
     const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
-    if (wpr == 0) return 1;
     LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
-    const unsigned groups = (unsigned)(((uint64_t)N * wpr + kBlock - 1) / kBlock);
 #define LM_CULL_SETUP(W_)                                                                                             \
-    hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3(groups), dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, \
-                       ray_list, bins, n_valid, acc, depth, app_cnt, p_end)
-    if (wpr == 1) LM_CULL_SETUP(1);
-    else if (wpr == 2) LM_CULL_SETUP(2);
-    else
+    hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3((unsigned)(((uint64_t)N * W_ + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, \
+                       *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt, p_end)
+    if (wpr == 1) {
+        LM_CULL_SETUP(1);
+    } else if (wpr == 2) {
+        LM_CULL_SETUP(2);
+    } else {
+        if (wpr == 0) {
+            const uint64_t n_words = ((uint64_t)N * (uint64_t)geom->S + 63) / 64;
+            const unsigned blocks = (unsigned)std::min<uint64_t>((n_words + kBlock - 1) / kBlock, 4096);
+            hipLaunchKernelGGL(k_zero_words, dim3(blocks), dim3(kBlock), 0, st, bitmap, n_words);
+        }
         hipLaunchKernelGGL(k_cull_rays_setup_serial, dim3((unsigned)(((uint64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                           st, *geom, rays, (uint32_t)N, (uint32_t)wpr, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth,
-                           app_cnt, p_end);
+                           st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt,
+                           p_end);
+    }
 #undef LM_CULL_SETUP
     LM_CHECK_LAUNCH("k_cull_rays_setup");
     return LM_OK;
