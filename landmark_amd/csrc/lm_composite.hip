@@ -11,6 +11,9 @@
 // A ray's slots are therefore contiguous and in sample order.
 // k_composite: one lane per ray sums weight * rgb over its slots, adds the white
 // background and clamps.
+// In the whole-chunk render the weights come from the marching kernel (density gather fused with
+// the transmittance walk); k_app_slots then builds the appearance list from the stored weights the
+// way k_weights' second pass does.  k_weights remains the stage-level form.
 //
 // Reference: raw2alpha (app/tools/utils.py:51-64), dists with a zero last interval
 // (app/models/gridnerf_sequential.py:457, 531-534), weight threshold (:479, :553) and the

@@ -8,6 +8,11 @@
 //   k_emit         per-word prefix and the ascending list of valid flat indices
 // The list order is the row-major order of the reference's boolean-mask indexing
 // (app/models/gridnerf_sequential.py:461-465, 472), so indices match it exactly.
+//
+// The whole-chunk render needs the decisions but no global order of the valid samples; it takes
+//   k_cull_rays_setup / k_cull_rays_setup_serial  one lane per (ray, word) or per ray: bitmap, a
+//       contiguous range of compact positions per ray, and the rays filed into the marching queue
+// which make bit-identical decisions (the same device functions of lm_common.h).
 #include <limits.h>
 
 #include <algorithm>
