@@ -112,7 +112,7 @@ struct Workspace {
     size_t total;
 };
 
-Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products) {
+Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products, float weight_thres) {
     Workspace w;
     size_t o = 0;
     auto take = [&](size_t bytes) {
@@ -121,8 +121,11 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products)
         return p;
     };
     const uint64_t total = (uint64_t)N * (uint64_t)S, n_words = (total + 63) / 64;
-    // every sample may be valid and (for S below 1/threshold) above the weight threshold
-    const uint64_t cap = total;
+    // Every sample may be valid.  A ray's weights are non-negative and sum to at most 1 (+ S * 1e-10 from the
+    // reference's cumulative-product guard), so at most 1 / threshold of them exceed the threshold.
+    uint64_t per_ray = (uint64_t)S;
+    if (weight_thres > 0.0f) per_ray = std::min<uint64_t>(per_ray, (uint64_t)(1.001 / (double)weight_thres) + 2);
+    const uint64_t cap = (uint64_t)N * per_ray;
     w.bitmap = (uint64_t *)take(n_words * 8);
     w.w_valid = (float *)take(total * 4);
     w.app_first = (uint32_t *)take((uint64_t)N * 4);
@@ -163,7 +166,7 @@ int check_model(const lm_model *m, int *K) {
 extern "C" size_t lm_render_workspace_bytes(const lm_model *m, int64_t N) {
     int K;
     if (check_model(m, &K) || N <= 0) return 0;
-    return carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m)).total;
+    return carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m), m->weight_thres).total;
 }
 
 extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
@@ -177,7 +180,7 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     const int S = m->geom.S;
     LM_REQUIRE((uint64_t)N * (uint64_t)S < (1ull << 32), "N*S does not fit 32-bit sample indices; split the chunk");
     const bool fused = lm_app_feat_supported(m) != 0;
-    Workspace w = carve((char *)workspace, N, S, K, !fused);
+    Workspace w = carve((char *)workspace, N, S, K, !fused, m->weight_thres);
     if (w.total > workspace_bytes)
         LM_FAIL(LM_ERR_WORKSPACE, "workspace has %zu bytes, %zu needed for N=%lld S=%d K=%d", workspace_bytes, w.total,
                 (long long)N, S, K);
