@@ -50,6 +50,15 @@
 #ifndef LM_MLPX2_NCB
 #define LM_MLPX2_NCB 1
 #endif
+#ifndef LM_MLPX2_NB
+#define LM_MLPX2_NB 1  // split mode: one accumulator block at a time keeps the wave inside 256 registers
+#endif
+#ifndef LM_MLPX2_PREFETCH
+#define LM_MLPX2_PREFETCH 0  // split mode: the second wave of the SIMD hides the input load, 16 registers are worth more
+#endif
+#ifndef LM_MLP16_NB1
+#define LM_MLP16_NB1 4  // 16-bit modes with one column block: row blocks per pass
+#endif
 
 namespace {
 
@@ -263,13 +272,7 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
     using frag = typename M::frag;
     constexpr int G = M::G, NP = M::NP;
     constexpr int T1 = kSlots1 / G, T2 = 64 / G;
-#ifndef LM_MLPX2_NB
-#define LM_MLPX2_NB 1  // split mode: one accumulator at a time keeps the wave inside 256 registers
-#endif
     // row blocks per pass: NB*NCB accumulators of 16 registers
-#ifndef LM_MLP16_NB1
-#define LM_MLP16_NB1 4
-#endif
     constexpr int NB = NCB == 1 ? (PREC == LM_MLP_F16X2 ? LM_MLPX2_NB : (PREC == LM_MLP_F32 ? 4 : LM_MLP16_NB1)) : 2;
     constexpr int PF = G == 1 ? 4 : 1;
     const unsigned h = lane >> 5;
@@ -424,9 +427,6 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
             raw[cb][15] = 0.0f;
         }
     };
-#ifndef LM_MLPX2_PREFETCH
-#define LM_MLPX2_PREFETCH 0  // split mode: the second wave of the SIMD hides the load, the 16 registers are worth more
-#endif
     // the next tile's inputs travel while this tile is multiplied
     constexpr bool kPrefetch = PREC != LM_MLP_F16X2 || LM_MLPX2_PREFETCH;
     float nxt[NCB][16];
