@@ -149,7 +149,7 @@ typedef struct lm_model {
 /* N_MARCHED: valid samples whose density was gathered (< N_VALID with early termination);
  * QUEUE: internal work-queue cursor; BINS..BINS+3: rays with valid samples, by how many they have
  * (>= 64, >= 32, >= 12, fewer): the marching queue hands out the long rays first. */
-enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_MARCHED = 2, LM_STAT_QUEUE = 3, LM_STAT_BINS = 4, LM_STAT_WORDS = 8 };
+enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_MARCHED = 2, LM_STAT_BINS = 4, LM_STAT_QUEUE = 8, LM_STAT_WORDS = 16 };
 
 int lm_abi_version(void);
 const char *lm_last_error(void);

@@ -14,7 +14,7 @@ SO_PATH = os.path.join(HERE, "liblandmark_hip.so")
 LM_MAX_PLANES = 12
 LM_N_STAGES = 6
 STAGE_NAMES = ["cull", "density_march", "app_list", "app_gather", "colour", "composite"]
-LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_N_MARCHED, LM_STAT_QUEUE, LM_STAT_BINS, LM_STAT_WORDS = 0, 1, 2, 3, 4, 8
+LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_N_MARCHED, LM_STAT_BINS, LM_STAT_QUEUE, LM_STAT_WORDS = 0, 1, 2, 4, 8, 16
 LM_F32, LM_F16, LM_U8, LM_CELLS = 0, 1, 2, 3
 LM_SAMPLER_AABB, LM_SAMPLER_HULL = 0, 1
 LM_ACT_SOFTPLUS, LM_ACT_RELU = 0, 1

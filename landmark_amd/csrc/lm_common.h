@@ -7,6 +7,7 @@
 #include "../../include/landmark_hip.h"
 
 #define LM_WAVE 64
+#define LM_XCDS 8  // accelerator dies, each with its own L2; workgroups are dealt to them round robin
 
 // Error plumbing: thread-local message, negative status.
 void lm_set_error(const char *fmt, ...);

@@ -215,11 +215,40 @@ __device__ __forceinline__ void footprint_products(const Footprint<T> &f, const 
     }
 }
 
-// NS samples at once (the marching kernel's look-ahead): the loads of all are issued before any
-// is used, so a ray's chain of dependent memory round trips is NS times shorter.  Same
-// operations per sample as density_sum, hence the same bits.
+// Value of v on lane n of this lane's quad (n is a constant after unrolling): one DPP move.
+__device__ __forceinline__ int quad_lane(int v, int n) {
+    switch (n & 3) {
+        case 0: return __builtin_amdgcn_update_dpp(0, v, 0x00, 0xf, 0xf, false);
+        case 1: return __builtin_amdgcn_update_dpp(0, v, 0x55, 0xf, 0xf, false);
+        case 2: return __builtin_amdgcn_update_dpp(0, v, 0xaa, 0xf, 0xf, false);
+        default: return __builtin_amdgcn_update_dpp(0, v, 0xff, 0xf, 0xf, false);
+    }
+}
+__device__ __forceinline__ float quad_lane(float v, int n) { return __int_as_float(quad_lane(__float_as_int(v), n)); }
+__device__ __forceinline__ int64_t quad_lane(int64_t v, int n) {
+    const uint32_t lo = (uint32_t)quad_lane((int)(uint32_t)v, n), hi = (uint32_t)quad_lane((int)(uint32_t)((uint64_t)v >> 32), n);
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ Taps2 quad_lane(const Taps2 &t, int n) {
+    Taps2 r;
+    r.o00 = quad_lane(t.o00, n); r.o01 = quad_lane(t.o01, n); r.o10 = quad_lane(t.o10, n); r.o11 = quad_lane(t.o11, n);
+    r.w00 = quad_lane(t.w00, n); r.w01 = quad_lane(t.w01, n); r.w10 = quad_lane(t.w10, n); r.w11 = quad_lane(t.w11, n);
+    return r;
+}
+__device__ __forceinline__ Taps1 quad_lane(const Taps1 &t, int n) {
+    Taps1 r;
+    r.o0 = quad_lane(t.o0, n); r.o1 = quad_lane(t.o1, n); r.w0 = quad_lane(t.w0, n); r.w1 = quad_lane(t.w1, n);
+    return r;
+}
+
+// NS samples of a quad at once (the marching kernel's look-ahead).  Lane n of the quad brings
+// the coordinates of sample n (lanes NS.. repeat) and works out that sample's footprints, one
+// sample per lane instead of every sample on every lane; the footprints then go round the quad
+// and each lane loads its quarter of the channels of all NS samples, every load issued before
+// the first use, so a ray's chain of dependent memory round trips is NS times shorter.  Same
+// operations per sample as density_sum, hence the same bits.  out[n] is valid on all four lanes.
 template <typename T, int NS>
-__device__ __forceinline__ void density_sum_n(const PlaneSet &ps, const float (*q)[4], unsigned qlane,
+__device__ __forceinline__ void density_sum_n(const PlaneSet &ps, const float *q_mine, unsigned qlane,
                                               const float *__restrict__ den_w, float *out) {
     constexpr int V = Vec<T>::V;
     float sum[NS];
@@ -228,13 +257,15 @@ __device__ __forceinline__ void density_sum_n(const PlaneSet &ps, const float (*
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
         const lm_plane &pl = ps.p[k];
+        Taps2 m2 = plane_taps(pl, pick(q_mine, pl.ax0), pick(q_mine, pl.ax1));
+        Taps1 m1 = line_taps(pl, pick(q_mine, pl.axl));
+        block_taps(pl, ps.nblk, q_mine, m2, m1);
         Taps2 t2[NS];
         Taps1 t1[NS];
 #pragma unroll
         for (int n = 0; n < NS; ++n) {
-            t2[n] = plane_taps(pl, pick(q[n], pl.ax0), pick(q[n], pl.ax1));
-            t1[n] = line_taps(pl, pick(q[n], pl.axl));
-            block_taps(pl, ps.nblk, q[n], t2[n], t1[n]);
+            t2[n] = quad_lane(m2, n);
+            t1[n] = quad_lane(m1, n);
         }
         for (int c = V * qlane; c < pl.C; c += V * kQuad) {
             Footprint<T> f[NS];
@@ -470,9 +501,18 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                                                   uint32_t *__restrict__ app_cnt, uint32_t *__restrict__ p_end_out,
                                                   uint32_t *__restrict__ n_marched) {
     const unsigned lane = lm_lane(), qlane = lane & 3u, leader = lane & ~3u;
+    // One cursor per XCD (workgroups go to the XCDs round robin): an XCD takes every n_queues-th
+    // granule of consecutive queue entries, so rays that are neighbours on screen march on the
+    // same XCD at the same time and meet in its L2.  Granules of 1024 rays when there are many,
+    // smaller ones for short queues so that every XCD still gets its share.
+    const uint32_t n_queues = gridDim.x < (unsigned)LM_XCDS ? gridDim.x : (unsigned)LM_XCDS;
+    const uint32_t my_q = blockIdx.x % n_queues;
+    uint32_t *my_queue = queue + my_q;
     uint32_t marched = 0;  // samples whose density this lane's quad gathered (statistics)
     // cumulative sizes of the four ray lists (long rays first)
     const uint32_t end0 = bins[0], end1 = end0 + bins[1], end2 = end1 + bins[2], n_active = end2 + bins[3];
+    const int log_n = 31 - __clz((int)(n_active | 1u));
+    const uint32_t granule_shift = (uint32_t)(log_n >= 16 ? 10 : log_n >= 10 ? log_n - 6 : 4);
     const int S = g.S;
     bool have = false, done = false;
     uint32_t r = 0, p = 0, cnt = 0;
@@ -487,10 +527,11 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
         if (need_mask) {
             const int first = __ffsll((unsigned long long)need_mask) - 1;
             uint32_t base = 0;
-            if ((int)lane == first) base = atomicAdd(queue, (uint32_t)__popcll(need_mask));
+            if ((int)lane == first) base = atomicAdd(my_queue, (uint32_t)__popcll(need_mask));
             base = __shfl(base, first);
             if (need) {
-                const uint32_t idx = base + (uint32_t)__popcll(need_mask & ((1ull << leader) - 1ull));
+                const uint32_t local = base + (uint32_t)__popcll(need_mask & ((1ull << leader) - 1ull));
+                const uint32_t idx = ((((local >> granule_shift) * n_queues + my_q)) << granule_shift) + (local & ((1u << granule_shift) - 1u));
                 if (idx >= n_active) {
                     done = true;
                 } else {
@@ -522,33 +563,47 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
             }
             bool finish = n_have == 0;
             if (!finish) {
-                int s_n[NS];
-                float z_n[NS], q[NS][4], f[NS];
+                // lane n of the quad prepares sample n: coordinates, footprints, and after the
+                // gather its alpha (missing samples repeat the first; their results are unused)
+                const int mine = (int)(qlane & (unsigned)(NS - 1));
+                uint64_t flat_m = flat[0];
+#pragma unroll
+                for (int n = 1; n < NS; ++n)
+                    if (mine == n && n < n_have) flat_m = flat[n];
+                const int s_m = (int)(flat_m - flat0);
+                const float z_m = lm_sample_z(g, rp, s_m);
+                float q_m[4], f[NS];
+                {
+                    float pt[3];
+                    lm_point(ray, z_m, pt);
+                    lm_normalise(g, pt, q_m);
+                    q_m[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q_m) : 0);
+                }
+                density_sum_n<T, NS>(ps, q_m, qlane, den_w, f);
+                marched += (uint32_t)n_have;
+                float f_m = f[0];
+#pragma unroll
+                for (int n = 1; n < NS; ++n)
+                    if (mine == n) f_m = f[n];
+                const float sig = activate(f_m, act, shift);
+                const float dist = (s_m + 1 < S) ? lm_sample_z(g, rp, s_m + 1) - z_m : 0.0f;
+                const float d2 = dist * distance_scale;
+                const float alpha_m = 1.0f - expf(-sig * d2);
+                float alpha_n[NS], z_n[NS];
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
-                    s_n[n] = (int)(flat[n < n_have ? n : 0] - flat0);  // missing samples repeat the first (result unused)
-                    z_n[n] = lm_sample_z(g, rp, s_n[n]);
-                    float pt[3];
-                    lm_point(ray, z_n[n], pt);
-                    lm_normalise(g, pt, q[n]);
-                    q[n][3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q[n]) : 0);
+                    alpha_n[n] = quad_lane(alpha_m, n);
+                    z_n[n] = quad_lane(z_m, n);
                 }
-                density_sum_n<T, NS>(ps, q, qlane, den_w, f);
-                marched += (uint32_t)n_have;
 #pragma unroll
                 for (int n = 0; n < NS; ++n) {
                     if (n >= n_have || finish) break;
-                    const int s = s_n[n];
-                    const float z = z_n[n];
-                    const float sig = activate(f[n], act, shift);
-                    const float dist = (s + 1 < S) ? lm_sample_z(g, rp, s + 1) - z : 0.0f;
-                    const float d2 = dist * distance_scale;
-                    const float alpha = 1.0f - expf(-sig * d2);
+                    const float alpha = alpha_n[n];
                     const float wgt = alpha * Tr;
                     Tr = Tr * ((1.0f - alpha) + 1e-10f);
                     if (qlane == 0) w_valid[p] = wgt;
                     acc += wgt;
-                    depth += wgt * z;
+                    depth += wgt * z_n[n];
                     cnt += wgt > weight_thres;
                     ++p;
                     finish = term_eps > 0.0f && Tr < term_eps;
