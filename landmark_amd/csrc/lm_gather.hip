@@ -76,23 +76,28 @@ struct Taps1 {
 
 __device__ __forceinline__ float unnorm(float c, int size) { return ((c + 1.0f) / 2.0f) * (float)(size - 1); }
 
+// Corner (y, x) outside the table has weight zero (grid_sample's zeros padding) and is read from
+// the nearest texel inside.  A row of the table has fewer than 2^31 elements (checked on the host).
 __device__ __forceinline__ Taps2 plane_taps(const lm_plane &pl, float cx, float cy) {
     const float ix = unnorm(cx, pl.W), iy = unnorm(cy, pl.H);
     const float fx = floorf(ix), fy = floorf(iy);
     float wx1 = ix - fx, wx0 = (fx + 1.0f) - ix, wy1 = iy - fy, wy0 = (fy + 1.0f) - iy;
     // clamp in float first: coordinates far outside the table must not overflow the int cast
-    int x0 = (int)fminf(fmaxf(fx, -2.0f), (float)pl.W), y0 = (int)fminf(fmaxf(fy, -2.0f), (float)pl.H);
-    int x1 = x0 + 1, y1 = y0 + 1;
-    if (x0 < 0 || x0 >= pl.W) wx0 = 0.0f;
-    if (x1 < 0 || x1 >= pl.W) wx1 = 0.0f;
-    if (y0 < 0 || y0 >= pl.H) wy0 = 0.0f;
-    if (y1 < 0 || y1 >= pl.H) wy1 = 0.0f;
-    x0 = min(max(x0, 0), pl.W - 1); x1 = min(max(x1, 0), pl.W - 1);
-    y0 = min(max(y0, 0), pl.H - 1); y1 = min(max(y1, 0), pl.H - 1);
+    const int x0 = (int)fminf(fmaxf(fx, -2.0f), (float)pl.W), y0 = (int)fminf(fmaxf(fy, -2.0f), (float)pl.H);
+    const int x1 = x0 + 1, y1 = y0 + 1;
+    if ((unsigned)x0 >= (unsigned)pl.W) wx0 = 0.0f;
+    if ((unsigned)x1 >= (unsigned)pl.W) wx1 = 0.0f;
+    if ((unsigned)y0 >= (unsigned)pl.H) wy0 = 0.0f;
+    if ((unsigned)y1 >= (unsigned)pl.H) wy1 = 0.0f;
+    const int x0c = min(max(x0, 0), pl.W - 1), x1c = min(max(x1, 0), pl.W - 1);
+    const int y0c = min(max(y0, 0), pl.H - 1), y1c = min(max(y1, 0), pl.H - 1);
+    const int row = pl.W * pl.C;
     Taps2 t;
-    const int64_t r0 = (int64_t)y0 * pl.W, r1 = (int64_t)y1 * pl.W;
-    t.o00 = (r0 + x0) * pl.C; t.o01 = (r0 + x1) * pl.C;
-    t.o10 = (r1 + x0) * pl.C; t.o11 = (r1 + x1) * pl.C;
+    const int dx = x1c != x0c ? pl.C : 0, dy = y1c != y0c ? row : 0;
+    t.o00 = (int64_t)y0c * row + x0c * pl.C;
+    t.o01 = t.o00 + dx;
+    t.o10 = t.o00 + dy;
+    t.o11 = t.o10 + dx;
     t.w00 = wx0 * wy0; t.w01 = wx1 * wy0; t.w10 = wx0 * wy1; t.w11 = wx1 * wy1;
     return t;
 }
@@ -125,6 +130,13 @@ __device__ __forceinline__ void block_taps(const lm_plane &pl, int nblk, const f
     t2.o00 += base; t2.o01 += base; t2.o10 += base; t2.o11 += base;
     t1.o0 = t1.o0 * nblk + blk * pl.C;
     t1.o1 = t1.o1 * nblk + blk * pl.C;
+}
+
+// Sum over the four lanes of a quad, on all four (DPP moves: partner 1 away, then 2 away).
+__device__ __forceinline__ float quad_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xb1, 0xf, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4e, 0xf, 0xf, false));
+    return v;
 }
 
 __device__ __forceinline__ float pick(const float *q, int ax) { return ax == 0 ? q[0] : (ax == 1 ? q[1] : q[2]); }
@@ -163,7 +175,7 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
     float sum = 0.0f;
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
-        const lm_plane &pl = ps.p[k];
+        const lm_plane pl = ps.p[k];
         Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
         Taps1 t1 = line_taps(pl, pick(q, pl.axl));
         block_taps(pl, ps.nblk, q, t2, t1);
@@ -180,8 +192,7 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
         }
         col += pl.C;
     }
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
+    sum = quad_sum(sum);
     return den_w ? fmaxf(sum, 0.0f) : sum;
 }
 
@@ -231,7 +242,12 @@ __device__ __forceinline__ int64_t quad_lane(int64_t v, int n) {
 }
 __device__ __forceinline__ Taps2 quad_lane(const Taps2 &t, int n) {
     Taps2 r;
-    r.o00 = quad_lane(t.o00, n); r.o01 = quad_lane(t.o01, n); r.o10 = quad_lane(t.o10, n); r.o11 = quad_lane(t.o11, n);
+    // the corners are less than 2^31 elements apart: one 64-bit offset and two 32-bit steps go round
+    const int dx = quad_lane((int)(t.o01 - t.o00), n), dy = quad_lane((int)(t.o10 - t.o00), n);
+    r.o00 = quad_lane(t.o00, n);
+    r.o01 = r.o00 + dx;
+    r.o10 = r.o00 + dy;
+    r.o11 = r.o10 + dx;
     r.w00 = quad_lane(t.w00, n); r.w01 = quad_lane(t.w01, n); r.w10 = quad_lane(t.w10, n); r.w11 = quad_lane(t.w11, n);
     return r;
 }
@@ -256,7 +272,7 @@ __device__ __forceinline__ void density_sum_n(const PlaneSet &ps, const float *q
     for (int n = 0; n < NS; ++n) sum[n] = 0.0f;
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
-        const lm_plane &pl = ps.p[k];
+        const lm_plane pl = ps.p[k];
         Taps2 m2 = plane_taps(pl, pick(q_mine, pl.ax0), pick(q_mine, pl.ax1));
         Taps1 m1 = line_taps(pl, pick(q_mine, pl.axl));
         block_taps(pl, ps.nblk, q_mine, m2, m1);
@@ -291,8 +307,7 @@ __device__ __forceinline__ void density_sum_n(const PlaneSet &ps, const float *q
 #pragma unroll
     for (int n = 0; n < NS; ++n) {
         float v = sum[n];
-        v += __shfl_xor(v, 1);
-        v += __shfl_xor(v, 2);
+        v = quad_sum(v);
         out[n] = den_w ? fmaxf(v, 0.0f) : v;
     }
 }
@@ -307,7 +322,7 @@ __device__ __forceinline__ float density_sum_fixed(const PlaneSet &ps, const flo
     constexpr int NG = (C + V * kQuad - 1) / (V * kQuad);
     float sum = 0.0f;
     for (int k = 0; k < ps.n; ++k) {
-        const lm_plane &pl = ps.p[k];
+        const lm_plane pl = ps.p[k];
         Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
         Taps1 t1 = line_taps(pl, pick(q, pl.axl));
         block_taps(pl, ps.nblk, q, t2, t1);
@@ -326,8 +341,7 @@ __device__ __forceinline__ float density_sum_fixed(const PlaneSet &ps, const flo
             }
         }
     }
-    sum += __shfl_xor(sum, 1);
-    sum += __shfl_xor(sum, 2);
+    sum = quad_sum(sum);
     return den_w ? fmaxf(sum, 0.0f) : sum;
 }
 
@@ -336,7 +350,7 @@ __device__ __forceinline__ void app_store(const PlaneSet &ps, const float *q, un
     constexpr int V = Vec<T>::V;
     int col = 0;
     for (int k = 0; k < ps.n; ++k) {
-        const lm_plane &pl = ps.p[k];
+        const lm_plane pl = ps.p[k];
         Taps2 t2 = plane_taps(pl, pick(q, pl.ax0), pick(q, pl.ax1));
         Taps1 t1 = line_taps(pl, pick(q, pl.axl));
         block_taps(pl, ps.nblk, q, t2, t1);
@@ -820,6 +834,7 @@ int lm_check_planes(const lm_plane *planes, int32_t n, int *dtype_out, int *K_ou
         LM_REQUIRE(p.plane && p.line, "plane %d: null table", k);
         LM_REQUIRE(lm_aligned16(p.plane) && lm_aligned16(p.line), "plane %d: tables must be 16-byte aligned", k);
         LM_REQUIRE(p.H > 0 && p.W > 0 && p.Len > 0, "plane %d: empty table", k);
+        LM_REQUIRE(p.C > 0 && (int64_t)p.W * p.C < ((int64_t)1 << 31), "plane %d: a row of more than 2^31 elements", k);
         LM_REQUIRE(p.dtype == planes[0].dtype, "planes must share one storage type");
         LM_REQUIRE(p.dtype == LM_F32 || p.dtype == LM_F16, "plane %d: unknown dtype %d", k, p.dtype);
         const int V = p.dtype == LM_F32 ? 4 : 8;
