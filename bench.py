@@ -146,6 +146,31 @@ def bench_frame(args, workload):
         ms_host_io = (time.perf_counter() - t0) / args.steps * 1e3
         assert torch.equal(rgb_h, rgb.cpu())
 
+    # the same frames with the chunks dealt to two streams (a workspace each): the compute-bound stages of one
+    # chunk run under the memory-bound stages of the other (reported beside the metric)
+    ms_two = None
+    if args.streams > 1 and n_chunks > 1:
+        streams = [torch.cuda.Stream() for _ in range(args.streams)]
+        slot_counters = torch.zeros((n_chunks, L.LM_STAT_WORDS), dtype=torch.int32, device=dev)
+        rgb2, depth2 = torch.empty_like(rgb), torch.empty_like(depth)
+
+        def frame_streams():
+            for ci in range(n_chunks):
+                sl = slice(ci * chunk, min((ci + 1) * chunk, N))
+                with torch.cuda.stream(streams[ci % args.streams]):
+                    model.render_into(rays[sl], rgb2[sl], depth2[sl], white_bg=True, counters=slot_counters[ci],
+                                      slot=ci % args.streams)
+
+        torch.cuda.synchronize()
+        frame_streams()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            frame_streams()
+        torch.cuda.synchronize()
+        ms_two = (time.perf_counter() - t0) / args.steps * 1e3
+        assert torch.equal(rgb2, rgb) and torch.equal(depth2, depth)
+
     cnt = counters.cpu().long() & 0xFFFFFFFF
     n_valid, n_app = int(cnt[:, L.LM_STAT_N_VALID].sum()), int(cnt[:, L.LM_STAT_N_APP].sum())
     n_marched = int(cnt[:, L.LM_STAT_N_MARCHED].sum())
@@ -215,6 +240,8 @@ def bench_frame(args, workload):
     }
     if ms_host_io is not None:
         out["ms_per_step_host_buffers"] = round(ms_host_io, 4)
+    if ms_two is not None:
+        out["ms_per_step_streams"] = {"streams": args.streams, "ms": round(ms_two, 4)}
     return out
 
 
@@ -352,6 +379,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--streams", type=int, default=2, help="also time the frame with its chunks dealt to this many streams")
     ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--planes", type=int, default=3, help="ndims of the c4 model (3 = XY,XZ,YZ; 1 = XY only)")
     ap.add_argument("--base", type=int, default=1024, help="base plane resolution of c4 (levels x1,x2,x4)")

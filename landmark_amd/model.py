@@ -110,7 +110,9 @@ class GridNeRFHIP:
         self._bias_code = {}
         self._pack_mlp(mlp_precision)
         # --- workspace cache (per-S geometry is cached in _geom_cache)
-        self._ws = None
+        self._ws = {}  # workspace per slot (one slot per stream that renders concurrently)
+        self._side_streams = []
+        self._slot_counters = []
         self.counters = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)
 
     # ------------------------------------------------------------------ construction helpers
@@ -287,17 +289,33 @@ class GridNeRFHIP:
             return int(self.p.n_importance)
         return int(N_samples) if N_samples > 0 else int(self.nSamples)
 
-    def workspace(self, n_rays: int, S: int) -> torch.Tensor:
+    def workspace(self, n_rays: int, S: int, slot: int = 0) -> torch.Tensor:
         """Device workspace for chunks of up to n_rays rays; grown on demand and reused
-        (the role of allocate_tensors, dist_render/kernel/cuda_render_extend.py:35-159)."""
+        (the role of allocate_tensors, dist_render/kernel/cuda_render_extend.py:35-159).
+        Renders that run concurrently on different streams take different slots."""
         m = self._model_struct(S, True)
         need = self.lib.lm_render_workspace_bytes(C.byref(m), n_rays)
         if need == 0:
             raise L.LandmarkError(self.lib.lm_last_error().decode())
-        if self._ws is None or self._ws.numel() < need:
-            self._ws = None
-            self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
-        return self._ws
+        ws = self._ws.get(slot)
+        if ws is None or ws.numel() < need:
+            self._ws[slot] = None
+            ws = self._ws[slot] = torch.empty(need, dtype=torch.uint8, device=self.device)
+        return ws
+
+    def slot_counters(self, slot: int) -> torch.Tensor:
+        """The counter block lm_render uses for a slot (slot 0: self.counters)."""
+        if slot == 0:
+            return self.counters
+        while len(self._slot_counters) < slot:
+            self._slot_counters.append(torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device))
+        return self._slot_counters[slot - 1]
+
+    def side_streams(self, n: int):
+        """n extra streams (default priority) for renders that overlap with the current stream's."""
+        while len(self._side_streams) < n:
+            self._side_streams.append(torch.cuda.Stream(device=self.device))
+        return self._side_streams[:n]
 
     # ------------------------------------------------------------------ reference interface
     def eval(self):
@@ -325,20 +343,22 @@ class GridNeRFHIP:
 
     __call__ = forward
 
-    def render_into(self, rays, rgb, depth, white_bg=True, N_samples=-1, counters=None, events=None):
-        """lm_render on device tensors the caller owns.  `counters`: int32[8] device tensor
+    def render_into(self, rays, rgb, depth, white_bg=True, N_samples=-1, counters=None, events=None, slot=0):
+        """lm_render on device tensors the caller owns.  `counters`: int32[LM_STAT_WORDS] device tensor
         receiving the chunk's sample counts; `events`: 7 recorded torch.cuda.Event objects
-        (enable_timing=True) re-recorded around the stages on the current stream."""
+        (enable_timing=True) re-recorded around the stages on the current stream.  Calls that may
+        run at the same time (different streams) must use different slots: a slot owns a workspace
+        and a counter block."""
         N = rays.shape[0]
         if N == 0:
             return
         S = self._samples_for(N_samples)
-        ws = self.workspace(N, S)
+        ws = self.workspace(N, S, slot)
         m = self._model_struct(S, white_bg)
         if events is not None:
             for i, e in enumerate(events):
                 m.events[i] = e.cuda_event
-        cnt = self.counters if counters is None else counters
+        cnt = self.slot_counters(slot) if counters is None else counters
         L.check(
             self.lib.lm_render(
                 C.byref(m), rays.data_ptr(), N, ws.data_ptr(), ws.numel(), rgb.data_ptr(), depth.data_ptr(),

@@ -93,30 +93,45 @@ def postprocess_rgba8(rgb_map, H, W):
 
 
 @torch.no_grad()
-def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 20, app_code=None, white_bg=True, depth=False):
+def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 20, app_code=None, white_bg=True, depth=False,
+                 streams=2):
     """Pose -> [H,W,4] uint8 image on the GPU: rays from the pose, the render in chunks, the RGBA8 conversion
     (the per-frame sequence of dist_render's inferer: generate_rays, renderer_fn, model_infer_postprocess;
     dist_render/ddp_infer/inferer_impl.py:143-170, nerf_inferer.py:345-378).  Rays are produced row by row, so the
     model is told the row length and chunks are cut at whole bands of 8 rows; nothing leaves the device.
-    With depth=True also returns the [H,W] depth map."""
+    The chunks are dealt to `streams` streams (the current one and side streams of the same priority, a workspace
+    each), so the compute-bound stages of one chunk run under the memory-bound stages of another; the current
+    stream continues after all of them.  With depth=True also returns the [H,W] depth map."""
     H, W = int(H), int(W)
     rays = generate_rays(single_pose, H, W, focal, device=gridnerf.device)
     N = H * W
     S = gridnerf._samples_for(-1)
-    if W % 8 == 0:
-        chunk = max(8 * W, int(chunk) // (8 * W) * (8 * W))
     while chunk * S >= 2**32:
         chunk //= 2
+    if W % 8 == 0:
+        chunk = max(8 * W, int(chunk) // (8 * W) * (8 * W))
     rgb = torch.empty((N, 3), dtype=torch.float32, device=gridnerf.device)
     dep = torch.empty((N,), dtype=torch.float32, device=gridnerf.device)
+    starts = list(range(0, N, chunk))
+    current = torch.cuda.current_stream(gridnerf.device)
+    side = gridnerf.side_streams(min(int(streams), len(starts)) - 1) if streams > 1 and len(starts) > 1 else []
+    gridnerf._set_app_code(gridnerf.mlp_precision, app_code)
+    if side:
+        ready = torch.cuda.Event()
+        ready.record(current)
+        for s in side:
+            s.wait_event(ready)
+    lanes = [current] + side
     saved = gridnerf.ray_row_length
     gridnerf.ray_row_length = W if W % 8 == 0 else 0
     try:
-        gridnerf._set_app_code(gridnerf.mlp_precision, app_code)
-        for start in range(0, N, chunk):
+        for i, start in enumerate(starts):
             sl = slice(start, min(start + chunk, N))
-            gridnerf.render_into(rays[sl], rgb[sl], dep[sl], white_bg=white_bg)
+            with torch.cuda.stream(lanes[i % len(lanes)]):
+                gridnerf.render_into(rays[sl], rgb[sl], dep[sl], white_bg=white_bg, slot=i % len(lanes))
     finally:
         gridnerf.ray_row_length = saved
+        for s in side:
+            current.wait_stream(s)
     image = postprocess_rgba8(rgb, H, W)
     return (image, dep.view(H, W)) if depth else image

@@ -494,6 +494,10 @@ def test_render_frame_from_pose(gpu_lib):
     assert diff.max().item() <= 1 and (diff > 0).float().mean().item() < 0.01
     assert (dep.cpu().reshape(-1) - ref["depth_map"]).abs().max().item() <= 2 * RGB_TOL_F32
     assert want[..., :3].min() < 250  # the scene is visible
+    # chunks dealt to one, two (the default) or three streams: the same bits
+    for n in (1, 3):
+        img_n, dep_n = render_frame(m, pose, H, W, chunk=20 * W, depth=True, streams=n)
+        assert torch.equal(img_n, img) and torch.equal(dep_n, dep)
 
 
 # ------------------------------------------------------------------------------------ occupancy volume from the model
