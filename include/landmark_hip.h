@@ -145,10 +145,12 @@ typedef struct lm_model {
     void *events[LM_N_STAGES + 1];
 } lm_model;
 
-/* Counters written by lm_render (device memory, 8 x uint32). */
+/* Counters written by lm_render (device memory, LM_STAT_WORDS x uint32). */
 /* N_MARCHED: valid samples whose density was gathered (< N_VALID with early termination);
- * QUEUE: internal work-queue cursor; BINS..BINS+3: rays with valid samples, by how many they have
- * (>= 64, >= 32, >= 12, fewer): the marching queue hands out the long rays first. */
+ * BINS..BINS+3: rays with valid samples, by how many they have (>= 64, >= 32, >= 12, fewer): the
+ * marching queue hands out the long rays first; QUEUE..QUEUE+7: internal cursors of that queue,
+ * one per XCD.  Two lm_render calls that may run at the same time (different streams) need a
+ * counter block and a workspace each. */
 enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_MARCHED = 2, LM_STAT_BINS = 4, LM_STAT_QUEUE = 8, LM_STAT_WORDS = 16 };
 
 int lm_abi_version(void);
