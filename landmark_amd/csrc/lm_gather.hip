@@ -29,21 +29,24 @@ struct PlaneSet {
     int nblk;  // > 0: block-stacked tables, planes [nblk][H][W][C], lines [Len][nblk][C]
 };
 
+// A lane's share of one texel: loaded as it is stored (fetch), converted to float where it is
+// used (unpack), so that loads in flight hold the stored width in registers and no conversion
+// waits for a load that other work could run under.
 template <typename T> struct Vec;
 template <> struct Vec<float> {
     using elem = float;
+    using raw = float4;
     static constexpr int V = 4;
-    __device__ static __forceinline__ void load(const float *p, float *o) {
-        float4 v = *reinterpret_cast<const float4 *>(p);
-        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
-    }
+    __device__ static __forceinline__ raw fetch(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+    __device__ static __forceinline__ void unpack(const raw &v, float *o) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
 };
 template <> struct Vec<__half> {
     using elem = __half;
+    using raw = uint4;
     static constexpr int V = 8;
-    __device__ static __forceinline__ void load(const __half *p, float *o) {
-        uint4 raw = *reinterpret_cast<const uint4 *>(p);
-        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+    __device__ static __forceinline__ raw fetch(const __half *p) { return *reinterpret_cast<const uint4 *>(p); }
+    __device__ static __forceinline__ void unpack(const raw &v, float *o) {
+        const __half2 *h = reinterpret_cast<const __half2 *>(&v);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float2 f = __half22float2(h[i]);
@@ -56,10 +59,11 @@ template <> struct Vec<__half> {
 struct Half4 {};
 template <> struct Vec<Half4> {
     using elem = __half;
+    using raw = uint2;
     static constexpr int V = 4;
-    __device__ static __forceinline__ void load(const __half *p, float *o) {
-        const uint2 raw = *reinterpret_cast<const uint2 *>(p);
-        const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+    __device__ static __forceinline__ raw fetch(const __half *p) { return *reinterpret_cast<const uint2 *>(p); }
+    __device__ static __forceinline__ void unpack(const raw &v, float *o) {
+        const __half2 *h = reinterpret_cast<const __half2 *>(&v);
         const float2 a = __half22float2(h[0]), b = __half22float2(h[1]);
         o[0] = a.x; o[1] = a.y; o[2] = b.x; o[3] = b.y;
     }
@@ -149,12 +153,11 @@ __device__ __forceinline__ void plane_products(const lm_plane &pl, const Taps2 &
     const E *P = reinterpret_cast<const E *>(pl.plane);
     const E *Ln = reinterpret_cast<const E *>(pl.line);
     float a[V], b[V], cc[V], d[V], l0[V], l1[V];
-    Vec<T>::load(P + t2.o00 + c, a);
-    Vec<T>::load(P + t2.o01 + c, b);
-    Vec<T>::load(P + t2.o10 + c, cc);
-    Vec<T>::load(P + t2.o11 + c, d);
-    Vec<T>::load(Ln + t1.o0 + c, l0);
-    Vec<T>::load(Ln + t1.o1 + c, l1);
+    const typename Vec<T>::raw ra = Vec<T>::fetch(P + t2.o00 + c), rb = Vec<T>::fetch(P + t2.o01 + c),
+                               rc = Vec<T>::fetch(P + t2.o10 + c), rd = Vec<T>::fetch(P + t2.o11 + c),
+                               r0 = Vec<T>::fetch(Ln + t1.o0 + c), r1 = Vec<T>::fetch(Ln + t1.o1 + c);
+    Vec<T>::unpack(ra, a); Vec<T>::unpack(rb, b); Vec<T>::unpack(rc, cc); Vec<T>::unpack(rd, d);
+    Vec<T>::unpack(r0, l0); Vec<T>::unpack(r1, l1);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
         float pv = a[i] * t2.w00;
@@ -199,29 +202,33 @@ __device__ __forceinline__ float density_sum(const PlaneSet &ps, const float *q,
 // The loads of plane_products and the arithmetic on what they return, as two steps, for callers
 // that want several footprints' loads in flight before the first use.
 template <typename T> struct Footprint {
-    float a[Vec<T>::V], b[Vec<T>::V], c[Vec<T>::V], d[Vec<T>::V], l0[Vec<T>::V], l1[Vec<T>::V];
+    typename Vec<T>::raw a, b, c, d, l0, l1;
 };
 template <typename T>
 __device__ __forceinline__ void footprint_load(const lm_plane &pl, const Taps2 &t2, const Taps1 &t1, int c, Footprint<T> &f) {
     using E = typename Vec<T>::elem;
     const E *P = reinterpret_cast<const E *>(pl.plane);
     const E *Ln = reinterpret_cast<const E *>(pl.line);
-    Vec<T>::load(P + t2.o00 + c, f.a);
-    Vec<T>::load(P + t2.o01 + c, f.b);
-    Vec<T>::load(P + t2.o10 + c, f.c);
-    Vec<T>::load(P + t2.o11 + c, f.d);
-    Vec<T>::load(Ln + t1.o0 + c, f.l0);
-    Vec<T>::load(Ln + t1.o1 + c, f.l1);
+    f.a = Vec<T>::fetch(P + t2.o00 + c);
+    f.b = Vec<T>::fetch(P + t2.o01 + c);
+    f.c = Vec<T>::fetch(P + t2.o10 + c);
+    f.d = Vec<T>::fetch(P + t2.o11 + c);
+    f.l0 = Vec<T>::fetch(Ln + t1.o0 + c);
+    f.l1 = Vec<T>::fetch(Ln + t1.o1 + c);
 }
 template <typename T>
 __device__ __forceinline__ void footprint_products(const Footprint<T> &f, const Taps2 &t2, const Taps1 &t1, float *prod) {
+    constexpr int V = Vec<T>::V;
+    float a[V], b[V], c[V], d[V], l0[V], l1[V];
+    Vec<T>::unpack(f.a, a); Vec<T>::unpack(f.b, b); Vec<T>::unpack(f.c, c); Vec<T>::unpack(f.d, d);
+    Vec<T>::unpack(f.l0, l0); Vec<T>::unpack(f.l1, l1);
 #pragma unroll
-    for (int i = 0; i < Vec<T>::V; ++i) {
-        float pv = f.a[i] * t2.w00;
-        pv = fmaf(f.b[i], t2.w01, pv);
-        pv = fmaf(f.c[i], t2.w10, pv);
-        pv = fmaf(f.d[i], t2.w11, pv);
-        const float lv = fmaf(f.l1[i], t1.w1, f.l0[i] * t1.w0);
+    for (int i = 0; i < V; ++i) {
+        float pv = a[i] * t2.w00;
+        pv = fmaf(b[i], t2.w01, pv);
+        pv = fmaf(c[i], t2.w10, pv);
+        pv = fmaf(d[i], t2.w11, pv);
+        const float lv = fmaf(l1[i], t1.w1, l0[i] * t1.w0);
         prod[i] = pv * lv;
     }
 }
