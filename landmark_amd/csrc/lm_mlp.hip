@@ -416,14 +416,18 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
             const uint64_t pc = p < M ? p : M - 1;
             const float *f = feat + pc * kAppDim;
             const float *vsrc = MODE == 0 ? view + pc * 3 : view + 6 * (size_t)(app_idx[pc] / (uint32_t)S) + 3;
+            // Half h holds rows row_of(v, 0) + 4 h: features up to row 23, then rows 24..26 (features,
+            // h = 0) or 28..30 (the view direction, h = 1); rows 27 and 31 are zero.  Two base
+            // addresses per lane and compile-time offsets instead of an address per load.
+            static_assert(row_of(0, 1) == row_of(0, 0) + 4 && row_of(11, 1) == 23 && row_of(12, 0) == 24 &&
+                              row_of(12, 1) == 28 && kAppDim == 27,
+                          "input rows per lane half");
+            const float *body = f + 4 * h;
+            const float *tail = h ? vsrc : f + 24;
 #pragma unroll
-            for (int v = 0; v < 15; ++v) {
-                // both halves' rows are compile-time constants: pick the address, load unconditionally
-                const int r0 = row_of(v, 0), r1 = row_of(v, 1);
-                const float *a0 = f + r0;
-                const float *a1 = r1 < kAppDim ? f + r1 : vsrc + (r1 - 28);
-                raw[cb][v] = *(h ? a1 : a0);
-            }
+            for (int v = 0; v < 12; ++v) raw[cb][v] = body[row_of(v, 0)];
+#pragma unroll
+            for (int v = 12; v < 15; ++v) raw[cb][v] = tail[v - 12];
             raw[cb][15] = 0.0f;
         }
     };

@@ -55,6 +55,11 @@ def test_argument_validation_returns_status_not_abort(lib):
     assert rc == -1 and b"null table" in lib.lm_last_error()
     assert lib.lm_gather_density_xyz(pl, 13, None, None, 10, None, None) == -1
     assert lib.lm_relayout_nchw_to_hwc(None, None, 4, 4, 4, 0, None) == -1
+    # a table row must stay below 2^31 elements: the kernels step between corners with 32-bit offsets
+    pl[0].plane = pl[0].line = 16
+    pl[0].H, pl[0].W, pl[0].Len, pl[0].C = 4, 1 << 26, 4, 32
+    rc = lib.lm_gather_density_xyz(pl, 1, None, None, 10, None, None)
+    assert rc == -1 and b"2^31" in lib.lm_last_error()
 
 
 def _host_model(S=128, C=48, n=3):
