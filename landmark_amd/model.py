@@ -303,6 +303,21 @@ class GridNeRFHIP:
             ws = self._ws[slot] = torch.empty(need, dtype=torch.uint8, device=self.device)
         return ws
 
+    # bytes of workspace a render may take when the library picks the chunk size itself
+    workspace_budget = 24 << 30
+
+    def preferred_chunk(self, n_rays: int, N_samples: int = -1) -> int:
+        """Rays per lm_render call when the caller leaves the choice to the library: up to 2^20
+        (large launches are what keeps the GPU busy: a 1080p frame in 4096-ray chunks takes 14
+        times as long as in two chunks), as many as `workspace_budget` and 32-bit sample indices allow."""
+        S = self._samples_for(N_samples)
+        m = self._model_struct(S, True)
+        probe = 1 << 16
+        per_ray = self.lib.lm_render_workspace_bytes(C.byref(m), probe) / probe
+        fit = int(self.workspace_budget / max(per_ray, 1.0))
+        cap = min(1 << 20, ((1 << 32) - 1) // S, max(fit, 4096))
+        return max(1, min(int(n_rays), cap))
+
     def slot_counters(self, slot: int) -> torch.Tensor:
         """The counter block lm_render uses for a slot (slot 0: self.counters)."""
         if slot == 0:
@@ -338,7 +353,10 @@ class GridNeRFHIP:
         N = rays.shape[0]
         rgb = torch.empty((N, 3), dtype=torch.float32, device=self.device)
         depth = torch.empty((N,), dtype=torch.float32, device=self.device)
-        self.render_into(rays, rgb, depth, white_bg=white_bg, N_samples=N_samples)
+        step = self.preferred_chunk(N, N_samples) if N else 1  # a call of any size: split where one launch cannot take it
+        for start in range(0, N, step):
+            sl = slice(start, min(start + step, N))
+            self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples)
         return {"rgb_map": rgb, "depth_map": depth}, {}
 
     __call__ = forward

@@ -13,13 +13,20 @@ import torch
 
 
 def renderer_fn(rays, gridnerf, chunk=4096, N_samples=-1, white_bg=True, is_train=False, device="cuda", idxs=None,
-                app_code=None):
+                app_code=None, exact_chunk=False):
     """Returns ({"rgb_map": [N,3], "depth_map": [N]}, {}).  `app_code` (dist_render's
-    per-frame appearance code, inferer_impl.py:144-145) is forwarded when given."""
+    per-frame appearance code, inferer_impl.py:144-145) is forwarded when given.
+    Rays are independent, so the result does not depend on how they are cut into chunks (bit for
+    bit); `chunk` bounds memory in the reference and is a lower bound here: a model that offers
+    `preferred_chunk` gets launches of that size (up to 2^20 rays within its workspace budget)
+    unless exact_chunk=True asks for the reference's slicing."""
     extra_kw = {} if app_code is None else {"app_code": app_code}
     all_ret = {}
     extra_loss = {}
     n_all = rays.shape[0]
+    chunk = int(chunk)
+    if not exact_chunk and idxs is None and n_all > chunk and hasattr(gridnerf, "preferred_chunk"):
+        chunk = max(chunk, gridnerf.preferred_chunk(n_all, N_samples))
     for ci in range(n_all // chunk + int(n_all % chunk > 0)):
         rays_chunk = rays[ci * chunk : (ci + 1) * chunk].to(device)
         if idxs is not None:

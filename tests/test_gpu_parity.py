@@ -7,6 +7,8 @@ The appearance mask (weight > 1e-3) derives from floats that are summed in a dif
 order than ATen does, so it may flip for weights within rounding of the threshold; such
 samples are excluded by an explicit band and counted.
 """
+import ctypes as C
+
 import pytest
 import torch
 
@@ -417,11 +419,21 @@ def test_chunk_drivers(gpu_lib):
     rays = scenes.pinhole_rays(40, 40, 40.0, scenes.sphere_pose(2.5, 5))
     m = _model(p)
     full, _ = m(rays)
-    for chunk in (1, 333, 4096):
-        ret, extra = renderer_fn(rays, m, chunk=chunk, device="cuda")
+    for chunk, exact in ((1, True), (333, True), (333, False), (4096, False)):
+        ret, extra = renderer_fn(rays, m, chunk=chunk, device="cuda", exact_chunk=exact)
         assert extra == {} and set(ret) == {"rgb_map", "depth_map"}
         # rays are independent: any chunking gives identical bits
         assert torch.equal(ret["rgb_map"], full["rgb_map"]) and torch.equal(ret["depth_map"], full["depth_map"])
+    # the library's own choice of chunk: everything at once here, bounded by the workspace budget and by
+    # 32-bit sample indices; a single call larger than that is split inside forward
+    assert m.preferred_chunk(rays.shape[0]) == rays.shape[0] and m.preferred_chunk(1 << 30) == 1 << 20
+    small = _model(p)
+    small.workspace_budget = 5000 * small.lib.lm_render_workspace_bytes(C.byref(small._model_struct(64, True)), 1 << 16) // (1 << 16)
+    more = scenes.pinhole_rays(80, 80, 80.0, scenes.sphere_pose(2.5, 5))
+    assert 4096 <= small.preferred_chunk(more.shape[0]) < more.shape[0]
+    split, _ = small(more)
+    whole, _ = m(more)
+    assert torch.equal(split["rgb_map"], whole["rgb_map"]) and torch.equal(split["depth_map"], whole["depth_map"])
     fused = MultiBlockParallelHIP()
     fused.allocate_tensors(m, 512)
     ret = fused.forward(rays[:512].cuda(), app_code=None, white_bg=True)
