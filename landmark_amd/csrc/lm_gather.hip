@@ -1039,15 +1039,15 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
                        dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,   \
                        p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,            \
                        m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched)
-    // few narrow fp16 planes: a round is short and light on registers, four samples per round keep more loads
-    // in flight (16.6 -> 14.3 ms on three 8192 x 8192 x 16 planes; with fp32 planes the registers cost more)
-    const bool deep = m->n_planes <= 4;
+    // Four samples per round: one per lane of the quad for the footprint arithmetic, 24 loads per lane and plane
+    // in flight, half as many dependent round trips per ray as with two (1080p frame, nine fp32 planes: 2.70 ->
+    // 2.50 ms although the kernel then holds 223 registers and two waves per SIMD instead of three).
     if (dtype == LM_F32) {
-        LM_MARCH(float, 2);
+        LM_MARCH(float, 4);
     } else if (c_max <= 16) {  // 16-byte loads would leave half of every quad idle
-        if (deep) LM_MARCH(Half4, 4); else LM_MARCH(Half4, 2);
+        LM_MARCH(Half4, 4);
     } else {
-        LM_MARCH(__half, 2);
+        LM_MARCH(__half, 4);
     }
 #undef LM_MARCH
     LM_CHECK_LAUNCH("k_march");

@@ -459,7 +459,7 @@ def test_row_length_hint_changes_nothing(gpu_lib, S, width):
 
 @pytest.mark.parametrize("fp16_tables,res", [(False, (1,)), (True, (1,)), (True, (1, 2))])
 def test_early_termination_bounds(gpu_lib, fp16_tables, res):
-    """fp32 planes march two samples per round, three narrow fp16 planes four, six of them two."""
+    """Rays stop up to three samples late (four are gathered per round); fp32 planes, three and six narrow fp16 planes."""
     p = _scene(S=128, resMode=res)
     if fp16_tables:
         p = O.to_fp16_features(p)
