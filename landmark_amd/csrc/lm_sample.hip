@@ -209,7 +209,9 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
 // word outside the box costs a few instructions and no wave waits at a barrier for a slower one
 // (with one lane per word the workgroup lasts as long as its slowest word).  Rays reach the queue
 // in a less regular order this way, which costs the march a little; with one or two words per ray
-// the kernel above is the better trade.
+// the kernel above is the better trade.  When a chunk has too few rays to fill the GPU with one lane
+// each, LPR neighbouring lanes share a ray and take every LPR-th word of it.
+template <int LPR>
 __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, const float *__restrict__ rays, uint32_t N,
                                                                    uint32_t row, uint64_t *__restrict__ bitmap,
                                                                    uint32_t *__restrict__ p_first,
@@ -219,7 +221,8 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
                                                                    float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
                                                                    uint32_t *__restrict__ p_end) {
     const unsigned lane = lm_lane();
-    const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;  // position in the visiting order
+    const unsigned sub = threadIdx.x % LPR;  // this lane's share of its ray's words
+    const uint64_t o = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / LPR;  // position in the visiting order
     const uint64_t r = o < N ? lm_ray_order((uint32_t)o, N, row) : o;
     uint32_t cnt = 0;
     if (r < N) {
@@ -229,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
         // the ray's samples are bits [flat0, flat1) of the bitmap: whole words are stored, a first or last word
         // shared with a neighbouring ray is merged into the (zeroed) bitmap
         const uint64_t flat0 = r * (uint64_t)g.S, flat1 = flat0 + (uint64_t)g.S;
-        for (uint64_t w = flat0 >> 6; w * 64 < flat1; ++w) {
+        for (uint64_t w = (flat0 >> 6) + sub; w * 64 < flat1; w += LPR) {
             const uint64_t lo = w * 64 > flat0 ? w * 64 : flat0, hi = (w + 1) * 64 < flat1 ? (w + 1) * 64 : flat1;
             const uint64_t bits = segment_bits(g, ray, rp, (int)(lo - flat0), (int)(hi - lo), (int)(lo & 63));
             if (hi - lo == 64) bitmap[w] = bits;
@@ -237,7 +240,10 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
             cnt += (uint32_t)__popcll(bits);
         }
     }
-    uint32_t incl = cnt;
+    // the ray's count on all of its lanes; its first lane speaks for it from here on
+#pragma unroll
+    for (int d = 1; d < LPR; d <<= 1) cnt += __shfl_xor(cnt, d);
+    uint32_t incl = sub == 0 ? cnt : 0;
 #pragma unroll
     for (int d = 1; d < LM_WAVE; d <<= 1) {
         const uint32_t y = __shfl_up(incl, d);
@@ -249,13 +255,13 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
         if (lane == 0) base = atomicAdd(n_valid, total);
         base = __shfl(base, 0);
     }
-    const bool any = cnt != 0;
-    if (r < N) {
+    const bool any = cnt != 0, mine = r < N && sub == 0;
+    if (mine) {
         const uint32_t first = base + incl - cnt;
         p_first[r] = first;
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
     }
-    lm_ray_enqueue(any && r < N, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
+    lm_ray_enqueue(any && mine, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
 }
 
 // words of the bitmap that two rays share must start at zero (sample counts that are not multiples of 64)
@@ -515,9 +521,22 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
             const unsigned blocks = (unsigned)std::min<uint64_t>((n_words + kBlock - 1) / kBlock, 4096);
             hipLaunchKernelGGL(k_zero_words, dim3(blocks), dim3(kBlock), 0, st, bitmap, n_words);
         }
-        hipLaunchKernelGGL(k_cull_rays_setup_serial, dim3((unsigned)(((uint64_t)N + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                           st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt,
-                           p_end);
+        // one lane per ray when the chunk fills the GPU that way, otherwise 2 .. 16 lanes per ray
+        const int words = (geom->S + 63) / 64;
+        int lpr = 1;
+        while (lpr < 16 && 2 * lpr <= words && (uint64_t)N * lpr < (uint64_t)lm_persistent_blocks(2) * kBlock) lpr *= 2;
+#define LM_CULL_SERIAL(L_)                                                                                           \
+    hipLaunchKernelGGL(k_cull_rays_setup_serial<L_>, dim3((unsigned)(((uint64_t)N * L_ + kBlock - 1) / kBlock)),         \
+                       dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, \
+                       depth, app_cnt, p_end)
+        switch (lpr) {
+            case 1: LM_CULL_SERIAL(1); break;
+            case 2: LM_CULL_SERIAL(2); break;
+            case 4: LM_CULL_SERIAL(4); break;
+            case 8: LM_CULL_SERIAL(8); break;
+            default: LM_CULL_SERIAL(16); break;
+        }
+#undef LM_CULL_SERIAL
     }
 #undef LM_CULL_SETUP
     LM_CHECK_LAUNCH("k_cull_rays_setup");

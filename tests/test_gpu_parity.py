@@ -333,7 +333,7 @@ def _check_render(p, rays, tol, S=-1, white_bg=True, **kw):
     d_dep = (out["depth_map"].cpu() - ref["depth_map"]).abs()
     assert d_rgb[ok].max().item() <= tol, f"rgb max diff {d_rgb[ok].max().item()}"
     assert d_dep[ok].max().item() <= tol, f"depth max diff {d_dep[ok].max().item()}"
-    assert int(band.sum()) <= max(2, rays.shape[0] // 500)
+    assert int(band.sum()) <= max(2, ref["weight"].numel() // 64000)  # a few in a million samples sit in the band
     if band.any():
         assert d_rgb[band].max().item() <= 2e-3
     return ref, out
@@ -358,9 +358,10 @@ def test_render_random_scenes(gpu_lib, opt, act, shift, res, ndims):
     assert ref["app_mask"].any(), "scene must exercise the colour network"
 
 
-@pytest.mark.parametrize("opt,S", [(1, 192), (1, 320), (0, 448), (1, 100)])
+@pytest.mark.parametrize("opt,S", [(1, 192), (1, 320), (0, 448), (1, 100), (1, 600), (0, 1100)])
 def test_render_other_sample_counts(gpu_lib, opt, S):
-    """Multiples of 64 beyond 128 / 256 take the one-launch cull with one lane per ray; anything else the scan path."""
+    """Sample counts other than 64 and 128 take the cull that walks a ray's bitmap words in one lane, or, for a
+    chunk as small as this one, in 2, 4, 8 or 16 lanes (3, 5, 7, 2, 10 and 18 words per ray here)."""
     p = _scene(opt=opt, S=S, shift=0.0, step_ratio=0.08, thre=0.0)
     rays = scenes.pinhole_rays(40, 40, 34.0, scenes.sphere_pose(2.5, 9))
     ref, _ = _check_render(p, rays, RGB_TOL_F32, S=S)
