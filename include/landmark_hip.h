@@ -29,7 +29,8 @@
 extern "C" {
 #endif
 
-#define LM_ABI_VERSION 1
+/* Changes whenever a struct, an enum value or the meaning of an argument does (2: 16-word counter block). */
+#define LM_ABI_VERSION 2
 #define LM_MAX_PLANES 12 /* ndims * len(resMode) */
 
 typedef enum lm_status {

@@ -14,6 +14,7 @@ SO_PATH = os.path.join(HERE, "liblandmark_hip.so")
 LM_MAX_PLANES = 12
 LM_N_STAGES = 6
 STAGE_NAMES = ["cull", "density_march", "app_list", "app_gather", "colour", "composite"]
+LM_ABI_VERSION = 2  # include/landmark_hip.h
 LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_N_MARCHED, LM_STAT_BINS, LM_STAT_QUEUE, LM_STAT_WORDS = 0, 1, 2, 4, 8, 16
 LM_F32, LM_F16, LM_U8, LM_CELLS = 0, 1, 2, 3
 LM_SAMPLER_AABB, LM_SAMPLER_HULL = 0, 1
@@ -102,7 +103,7 @@ def load() -> C.CDLL:
     for name, (res, args) in SYMBOLS.items():
         fn = getattr(lib, name)  # AttributeError if the header and the library disagree
         fn.restype, fn.argtypes = res, args
-    if lib.lm_abi_version() != 1:
+    if lib.lm_abi_version() != LM_ABI_VERSION:
         raise LandmarkError(f"ABI version mismatch: library reports {lib.lm_abi_version()}")
     _lib = lib
     return lib
