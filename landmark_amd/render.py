@@ -88,27 +88,39 @@ def generate_rays(single_pose, H, W, focal=None, device="cuda"):
     return rays
 
 
-def postprocess_rgba8(rgb_map, H, W):
+def pinned_image(H, W):
+    """Page-locked host buffer for one [H,W,4] uint8 frame (allocated pinned; reuse it across frames)."""
+    return torch.empty((int(H), int(W), 4), dtype=torch.uint8, pin_memory=True)
+
+
+def postprocess_rgba8(rgb_map, H, W, host_image=None):
     """[H,W,4] uint8 image (alpha 255) from rgb in [0,1]
-    (model_infer_postprocess, dist_render/ddp_infer/nerf_inferer.py:366-370)."""
+    (model_infer_postprocess, dist_render/ddp_infer/nerf_inferer.py:366-370).  With `host_image` (from
+    pinned_image) the frame is also copied there on the current stream without blocking, the reference's
+    pinned device-to-host step (nerf_inferer.py:371-374); it is complete once the stream is synchronised."""
     from . import _lib as L
 
     rgb = rgb_map.contiguous()
     out = torch.empty((int(H), int(W), 4), dtype=torch.uint8, device=rgb.device)
     L.check(L.load().lm_rgba8(rgb.data_ptr(), rgb.shape[0], out.data_ptr(), L.current_stream()), "lm_rgba8")
+    if host_image is not None:
+        if not host_image.is_pinned() or host_image.shape != out.shape or host_image.dtype != torch.uint8:
+            raise ValueError("host_image must be a pinned uint8 tensor of shape [H,W,4]")
+        host_image.copy_(out, non_blocking=True)
     return out
 
 
 @torch.no_grad()
 def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 20, app_code=None, white_bg=True, depth=False,
-                 streams=2):
+                 streams=2, host_image=None):
     """Pose -> [H,W,4] uint8 image on the GPU: rays from the pose, the render in chunks, the RGBA8 conversion
     (the per-frame sequence of dist_render's inferer: generate_rays, renderer_fn, model_infer_postprocess;
     dist_render/ddp_infer/inferer_impl.py:143-170, nerf_inferer.py:345-378).  Rays are produced row by row, so the
     model is told the row length and chunks are cut at whole bands of 8 rows; nothing leaves the device.
     The chunks are dealt to `streams` streams (the current one and side streams of the same priority, a workspace
     each), so the compute-bound stages of one chunk run under the memory-bound stages of another; the current
-    stream continues after all of them.  With depth=True also returns the [H,W] depth map."""
+    stream continues after all of them.  With depth=True also returns the [H,W] depth map; with `host_image`
+    (pinned_image) the frame is also copied to the host without blocking."""
     H, W = int(H), int(W)
     rays = generate_rays(single_pose, H, W, focal, device=gridnerf.device)
     N = H * W
@@ -140,5 +152,5 @@ def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 20, app_cod
         gridnerf.ray_row_length = saved
         for s in side:
             current.wait_stream(s)
-    image = postprocess_rgba8(rgb, H, W)
+    image = postprocess_rgba8(rgb, H, W, host_image)
     return (image, dep.view(H, W)) if depth else image

@@ -507,6 +507,14 @@ def test_render_frame_from_pose(gpu_lib):
     assert diff.max().item() <= 1 and (diff > 0).float().mean().item() < 0.01
     assert (dep.cpu().reshape(-1) - ref["depth_map"]).abs().max().item() <= 2 * RGB_TOL_F32
     assert want[..., :3].min() < 250  # the scene is visible
+    # the pinned device-to-host step of the serving loop
+    from landmark_amd.render import pinned_image
+    host = pinned_image(H, W)
+    render_frame(m, pose, H, W, chunk=20 * W, host_image=host)
+    torch.cuda.current_stream().synchronize()
+    assert torch.equal(host, img.cpu())
+    with pytest.raises(ValueError):
+        render_frame(m, pose, H, W, host_image=torch.empty((H, W, 4), dtype=torch.uint8))
     # chunks dealt to one, two (the default) or three streams: the same bits
     for n in (1, 3):
         img_n, dep_n = render_frame(m, pose, H, W, chunk=20 * W, depth=True, streams=n)
