@@ -368,6 +368,35 @@ def test_render_other_sample_counts(gpu_lib, opt, S):
     assert ref["app_mask"].any()
 
 
+def test_render_configuration_sweep(gpu_lib):
+    """Forty seeded random configurations (sampler, sample count, levels, plane orientations, table storage,
+    activation, occupancy threshold, ragged ray counts) against the oracle: the combinations the fixed cases leave out."""
+    import random
+
+    rnd = random.Random(1234)
+    for it in range(40):
+        opt = rnd.choice([0, 1])
+        S = rnd.choice([16, 37, 64, 100, 128, 200, 256, 330])
+        res = rnd.choice([(1,), (1, 2), (1, 2, 4)])
+        ndims = rnd.choice([1, 2, 3])
+        fp16 = rnd.random() < 0.35
+        act = rnd.choice(["softplus", "relu"])
+        shift = rnd.choice([0.0, -1.0])
+        thre = rnd.choice([0.0, 0.0, 0.5])
+        mask = rnd.random() < 0.8
+        w, h, cut, seed = rnd.randint(3, 70), rnd.randint(3, 70), rnd.randint(0, 5), rnd.randint(0, 1000)
+        p = _scene(seed=seed, opt=opt, S=S, thre=thre, shift=shift, with_mask=mask, resMode=res, ndims=ndims,
+                   fea2denseAct=act, step_ratio=0.25 if opt == 0 else 2.0)
+        if fp16:
+            p = O.to_fp16_features(p)
+        rays = scenes.pinhole_rays(w, h, 0.8 * max(w, h), scenes.sphere_pose(2.5, seed % 17))[cut:]
+        try:
+            _check_render(p, rays, RGB_TOL_16 if fp16 else RGB_TOL_F32, S=S if opt == 0 else -1, mlp_precision="f16x2")
+        except AssertionError as e:
+            raise AssertionError(f"configuration {it}: opt {opt} S {S} res {res} ndims {ndims} fp16 {fp16} act {act} "
+                                 f"shift {shift} thre {thre} mask {mask} {w}x{h} cut {cut} seed {seed}: {e}") from e
+
+
 def test_appearance_embedding_and_density_projection(gpu_lib):
     """encode_app (latent folded into the first layer's bias, switched per call) and
     nonlinear_density against the oracle."""
