@@ -32,13 +32,29 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0, "bf16": 2500.0, "f16x2": 2500.0}
 MLP_FLOP_PER_ROW = 2 * (150 * 128 + 128 * 128 + 128 * 3)
-# HBM-side bytes per launch (L2 misses: FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc runs, scaled
-# by the factors a plain copy of known size gave: 2.00 and 1.00) of the default workload's gather
-# kernels at the default chunk size; any other configuration reports null.
-MEASURED_TRAFFIC = {
-    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_app_feat"): 16.42e9 + 0.42e9,
-    ("c4_1080p_multires_P3_base1024_shift0", 1044480, "k_march"): 7.63e9 + 0.08e9,
-}
+PROFILE_DIR = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(workload, chunk, mlp, term, kernel):
+    """HBM-side bytes per launch of `kernel` as the rocprofv3 counter runs summarised under profiles/ measured
+    them, or None.  A summary carries one line per kernel of the form
+        bench-traffic: workload=<name> chunk=<rays> mlp=<mode> term_eps=<auto|value> kernel=<k> fetch_bytes=<n> write_bytes=<n>
+    (FETCH_SIZE and WRITE_SIZE per dispatch, scaled by the factors a copy of known size gave in the same runs).
+    Returns (bytes, "file:line") for the first line that names this exact configuration."""
+    if not os.path.isdir(PROFILE_DIR):
+        return None
+    for fn in sorted(os.listdir(PROFILE_DIR)):
+        if not fn.endswith(".txt"):
+            continue
+        with open(os.path.join(PROFILE_DIR, fn)) as f:
+            for ln, line in enumerate(f, 1):
+                if not line.startswith("bench-traffic:"):
+                    continue
+                kv = dict(tok.split("=", 1) for tok in line.split()[1:] if "=" in tok)
+                if (kv.get("workload") == workload and kv.get("chunk") == str(chunk) and kv.get("mlp") == mlp
+                        and kv.get("term_eps") == term and kv.get("kernel") == kernel):
+                    return float(kv["fetch_bytes"]) + float(kv["write_bytes"]), f"profiles/{fn}:{ln}"
+    return None
 
 
 def log(*a):
@@ -50,6 +66,40 @@ def plane_bytes_per_sample(planes):
 
 
 # ----------------------------------------------------------------------------------------
+def frame_chunks(model, N, S, W, want, row_hint=True):
+    """Rays per lm_render call: as asked, within 32-bit sample indices, whole bands of 8 image rows when the
+    rays are an image's pixels (the library then visits them in 8 x 8 tiles)."""
+    chunk = min(want, N)
+    while chunk * S >= 2**32:
+        chunk //= 2
+    model.ray_row_length = 0
+    if row_hint and W % 8 == 0:
+        model.ray_row_length = W
+        chunk = max(8 * W, chunk // (8 * W) * (8 * W))
+    return chunk
+
+
+def time_frames(model, rays, rgb, depth, chunk, steps, warmup, counters=None, events=None):
+    """ms per frame over `steps` frames on the current stream (wall clock between two synchronisations)."""
+    N = rays.shape[0]
+    n_chunks = (N + chunk - 1) // chunk
+
+    def frame(ev=None):
+        for ci in range(n_chunks):
+            sl = slice(ci * chunk, min((ci + 1) * chunk, N))
+            model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=None if counters is None else counters[ci],
+                              events=None if ev is None else ev[ci])
+
+    for _ in range(warmup):
+        frame()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        frame(None if events is None else events[k])
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e3
+
+
 def bench_frame(args, workload):
     from landmark_amd import _lib as L
     from landmark_amd import scenes
@@ -57,11 +107,18 @@ def bench_frame(args, workload):
 
     dev = "cuda:0"
     t0 = time.time()
+    app_code = None
     if workload == "c4":
         p = scenes.c4_scene(P=args.planes, base=args.base, device=dev, density_shift=args.density_shift)
         H, W = args.height, args.width
         rays = scenes.c4_rays(H, W, frame=args.frame, device=dev)
         name = f"c4_1080p_multires_P{args.planes}_base{args.base}_shift{args.density_shift:g}"
+    elif workload == "prod":
+        p = scenes.production_scene(base=args.base, step_ratio=args.step_ratio, device=dev, density_shift=args.density_shift)
+        H, W = args.height, args.width
+        rays = scenes.c4_rays(H, W, frame=args.frame, device=dev)
+        name = f"prod_1080p_aabb_sampler_P1_L3_base{args.base}_step{args.step_ratio:g}_encodeapp_nonlinear"
+        app_code = 3
     elif workload == "c1":
         p = scenes.c1_scene(dense=args.density_shift == 0.0, device=dev)
         H, W = 400, 400
@@ -80,23 +137,18 @@ def bench_frame(args, workload):
     term_eps = 1e-4 / float(p.near_far[1]) if term_auto else float(args.term_eps)
     args.term_eps = term_eps
     model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=term_eps)
+    model._set_app_code(args.mlp, app_code)
     torch.cuda.synchronize()
     log(f"[bench] scene {name} built in {time.time() - t0:.1f}s; tables "
         f"{sum(t.numel() * t.element_size() for t in model._tables) / 1e9:.2f} GB")
     N = rays.shape[0]
     S = model._samples_for(-1)
-    chunk = min(args.chunk, N)
-    while chunk * S >= 2**32:
-        chunk //= 2
-    if not args.no_row_hint and W % 8 == 0:
-        # the rays are the frame's pixels row by row: tell the library, and cut chunks at whole bands of 8 rows
-        model.ray_row_length = W
-        chunk = max(8 * W, chunk // (8 * W) * (8 * W))
+    chunk = frame_chunks(model, N, S, W, args.chunk, not args.no_row_hint)
     n_chunks = (N + chunk - 1) // chunk
     rgb = torch.empty((N, 3), device=dev)
     depth = torch.empty((N,), device=dev)
     counters = torch.zeros((n_chunks, L.LM_STAT_WORDS), dtype=torch.int32, device=dev)
-    model.workspace(chunk, S)
+    ws = model.workspace(chunk, S)
     n_ev = L.LM_N_STAGES + 1
     events = [[[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(n_chunks)] for _ in range(args.steps)]
     for per_step in events:
@@ -104,21 +156,13 @@ def bench_frame(args, workload):
             for e in per_chunk:
                 e.record()  # creates the underlying hipEvent handle
 
-    def frame(ev=None):
+    # ---- the timed region: inputs resident, `steps` frames on one stream
+    ms_step = time_frames(model, rays, rgb, depth, chunk, args.steps, args.warmup, counters, events)
+
+    def frame_plain():
         for ci in range(n_chunks):
             sl = slice(ci * chunk, min((ci + 1) * chunk, N))
-            model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci],
-                              events=None if ev is None else ev[ci])
-
-    for _ in range(args.warmup):
-        frame()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        frame(events[k])
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_step = dt / args.steps * 1e3
+            model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci])
 
     # the same frames when the boundary hands over host buffers: rays from pinned host memory, rgb and depth back to
     # it, copies and kernels on the one stream (reported beside the metric, never as the metric)
@@ -170,10 +214,14 @@ def bench_frame(args, workload):
         torch.cuda.synchronize()
         ms_two = (time.perf_counter() - t0) / args.steps * 1e3
         assert torch.equal(rgb2, rgb) and torch.equal(depth2, depth)
+        del rgb2, depth2
 
     cnt = counters.cpu().long() & 0xFFFFFFFF
     n_valid, n_app = int(cnt[:, L.LM_STAT_N_VALID].sum()), int(cnt[:, L.LM_STAT_N_APP].sum())
     n_marched = int(cnt[:, L.LM_STAT_N_MARCHED].sum())
+    overflow = int(cnt[:, L.LM_STAT_OVERFLOW].sum()) if hasattr(L, "LM_STAT_OVERFLOW") else 0
+    if overflow:
+        raise RuntimeError(f"{overflow} rays did not fit the workspace capacity: the timed frames are incomplete")
     stage_ms = [0.0] * L.LM_N_STAGES  # per frame, averaged over steps
     for per_step in events:
         for per_chunk in per_step:
@@ -183,13 +231,18 @@ def bench_frame(args, workload):
     launches = n_chunks  # one launch of each stage kernel per chunk
     dens_B = plane_bytes_per_sample(model._density) + 4  # + weight out
     app_B = plane_bytes_per_sample(model._app) + 4 + 27 * 4  # + index in, projected features out
+    basis_flop = 2 * model.K_app * 27  # basis_mat runs inside the appearance gather
     stages = {}
     for i, nm in enumerate(L.STAGE_NAMES):
         stages[nm] = {"ms_per_frame": round(stage_ms[i], 4)}
+    # GB/s figures of the gathers are in gather-convention bytes: every corner load of every sample, no reuse
     stages["density_march"].update(bytes_per_sample=dens_B, samples=n_marched,
-                                   GBps=round(n_marched * dens_B / (stage_ms[1] * 1e-3) / 1e9, 1))
-    stages["app_gather"].update(bytes_per_sample=app_B, GBps=round(n_app * app_B / max(stage_ms[3], 1e-9) / 1e6, 1))
-    stages["colour"].update(TFLOPs=round(n_app * (MLP_FLOP_PER_ROW + 2 * model.K_app * 27) / max(stage_ms[4], 1e-9) / 1e9, 2))
+                                   convention_GBps=round(n_marched * dens_B / max(stage_ms[1], 1e-9) / 1e6, 1))
+    stages["app_gather"].update(bytes_per_sample=app_B, samples=n_app,
+                                convention_GBps=round(n_app * app_B / max(stage_ms[3], 1e-9) / 1e6, 1),
+                                basis_TFLOPs=round(n_app * basis_flop / max(stage_ms[3], 1e-9) / 1e9, 2))
+    stages["colour"].update(rows=n_app, TFLOPs=round(n_app * MLP_FLOP_PER_ROW / max(stage_ms[4], 1e-9) / 1e9, 2),
+                            frac_of_mfma_peak=round(n_app * MLP_FLOP_PER_ROW / max(stage_ms[4], 1e-9) / 1e9 / MFMA_PEAK_TFLOPS[args.mlp], 4))
     # occupancy lookups: 1 byte per sample from the cell table (8 x 4 bytes with a float volume), upper bound
     # every sample; 1 bit per sample and 24 bytes per ray besides
     cull_B = (1 if model._vol_dtype == L.LM_CELLS else 32 if model._vol is not None else 0) + 0.125
@@ -201,27 +254,38 @@ def bench_frame(args, workload):
     # dominant kernel -> roofline object
     cand = {"density_march": stage_ms[1], "app_gather": stage_ms[3], "colour": stage_ms[4]}
     dom = max(cand, key=cand.get)
+    avg_ms = cand[dom] / launches
     if dom == "colour":
         ach = stages["colour"]["TFLOPs"]
         peak = MFMA_PEAK_TFLOPS[args.mlp]
         roof = {"kernel": "k_mlp", "bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s",
                 "frac": round(ach / peak, 4), "traffic": None}
     else:
-        ach = stages[dom]["GBps"]
-        roof = {"kernel": "k_march" if dom == "density_march" else "k_app_feat", "bound": "hbm", "achieved": ach,
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None}
-    if roof["bound"] == "hbm":
-        roof["note"] = ("achieved = gather-convention bytes (every corner load of every sample, no reuse between samples) "
-                        "per launch / launch time; traffic = counter-derived HBM-side bytes of the same launch")
-    roof["avg_launch_ms"] = round(cand[dom] / launches, 4)
+        kernel = "k_march" if dom == "density_march" else "k_app_feat"
+        conv = stages[dom]["convention_GBps"]
+        found = measured_traffic(name, chunk, args.mlp, "auto" if term_auto else f"{term_eps:g}", kernel) \
+            if int(model.ray_row_length) == W else None
+        roof = {"kernel": kernel, "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "convention": "gather, no reuse: every corner load of every sample counted, line tables excluded",
+                "convention_bytes_per_launch": round(stages[dom]["samples"] * stages[dom]["bytes_per_sample"] / launches),
+                "convention_GBps": conv}
+        if found:
+            # bytes the launch moved past the L2 (rocprofv3 counters, summarised under profiles/) / its duration here
+            roof["traffic"], roof["traffic_source"] = found
+            roof["achieved"] = round(found[0] / (avg_ms * 1e-3) / 1e9, 1)
+            roof["frac"] = round(roof["achieved"] / HBM_PEAK_GBS, 4)
+            roof["basis"] = "counter-derived HBM-side bytes per launch / launch duration measured in this run"
+        else:
+            # no counter figure for this configuration: the convention rate is an upper bound of the HBM rate (texels
+            # shared by neighbouring samples are counted once per sample), so it is no fraction of the peak
+            roof["traffic"] = None
+            roof["achieved"] = conv
+            roof["frac"] = round(conv / HBM_PEAK_GBS, 4) if conv <= HBM_PEAK_GBS else None
+            roof["basis"] = "gather-convention bytes / launch duration (no counter run covers this configuration)"
+    roof["avg_launch_ms"] = round(avg_ms, 4)
     roof["launches_per_frame"] = launches
-    measured = term_auto and args.mlp == "f16x2" and int(model.ray_row_length) == W
-    roof["traffic"] = MEASURED_TRAFFIC.get((name, chunk, roof["kernel"])) if measured else None
-    if roof["traffic"]:
-        # the same launch priced by its counter-derived L2-miss traffic instead of the gather-convention bytes
-        roof["traffic_GBps"] = round(roof["traffic"] / (roof["avg_launch_ms"] * 1e-3) / 1e9, 1)
 
-    cpu, parity = cpu_baseline_frame(args, p, rays, rgb, depth, H, W)
+    cpu, parity = cpu_baseline_frame(args, p, rays, rgb, depth, H, W, app_code)
     mrays = N / (ms_step * 1e-3) / 1e6
     out = {
         "metric": "render_throughput", "value": round(mrays, 3), "unit": "Mrays/s", "n_gpus": 1,
@@ -229,29 +293,41 @@ def bench_frame(args, workload):
         "scaling": "weak", "vs_baseline": None, "dtype": ("f16" if p.app_plane[0].dtype == torch.float16 else "f32") + ("" if args.mlp == "f32" else f"+{args.mlp}-mlp"),
         "data": "synthetic",
         "config": {"workload": name, "rays": N, "samples_per_ray": S, "chunk_rays": chunk, "ray_row_hint": int(model.ray_row_length), "mlp": args.mlp,
-                   "term_eps": args.term_eps, "valid_samples": n_valid, "marched_samples": n_marched, "app_samples": n_app},
+                   "term_eps": args.term_eps, "valid_samples": n_valid, "marched_samples": n_marched, "app_samples": n_app,
+                   "workspace_GB": round(ws.numel() / 1e9, 3)},
         "frames_per_s": round(1e3 / ms_step, 3), "mpixel_per_s": round(mrays, 3),
-        # feature gather: gather-convention bytes per second of both gather kernels, and the dominant one's
-        # counter-derived HBM traffic rate against the HBM peak (null where it was not measured)
-        "gather_algorithmic_GBps": {"density": stages["density_march"]["GBps"], "appearance": stages["app_gather"]["GBps"]},
-        "gather_hbm_GBps": roof.get("traffic_GBps"),
-        "gather_frac_of_hbm_peak": round(roof["traffic_GBps"] / HBM_PEAK_GBS, 4) if roof.get("traffic_GBps") else None,
         "stages": stages, "roofline": roof, "cpu_baseline": cpu, "parity": parity,
     }
     if ms_host_io is not None:
         out["ms_per_step_host_buffers"] = round(ms_host_io, 4)
     if ms_two is not None:
         out["ms_per_step_streams"] = {"streams": args.streams, "ms": round(ms_two, 4)}
+    if workload == "c4" and not args.no_extra:
+        # the same frame in two more settings, timed in this run after the region above (never `value`):
+        # the reference-semantics mode (fp32 matrix products, no early termination) and the one-orientation model
+        steps = max(3, args.steps // 2)
+        model.mlp_precision, model.term_eps = "f32", 0.0
+        out["ms_per_step_exact"] = {"mlp": "f32", "term_eps": 0.0,
+                                    "ms": round(time_frames(model, rays, rgb, depth, chunk, steps, 2), 4)}
+        del model
+        torch.cuda.empty_cache()
+        if args.planes != 1:
+            p1 = scenes.c4_scene(P=1, base=args.base, device=dev, density_shift=args.density_shift)
+            m1 = GridNeRFHIP(p1, device=dev, mlp_precision=args.mlp, term_eps=term_eps, release_source=True)
+            c1 = frame_chunks(m1, N, S, W, args.chunk, not args.no_row_hint)
+            out["ms_per_step_P1"] = {"workload": f"c4_1080p_multires_P1_base{args.base}_shift{args.density_shift:g}",
+                                     "ms": round(time_frames(m1, rays, rgb, depth, c1, steps, 2), 4)}
     return out
 
 
-def cpu_baseline_frame(args, p, rays, rgb, depth, H, W):
+def cpu_baseline_frame(args, p, rays, rgb, depth, H, W, app_code=None):
     """The CPU oracle on a bounded sample of the frame (evenly spaced scan-lines)."""
     if args.no_cpu:
         return None, None
     from oracle import gridnerf_oracle as O
 
-    rows = max(1, min(H, args.cpu_rows))
+    S = p.n_importance if p.sampling_opt else p.nSamples
+    rows = max(1, min(H, args.cpu_rows * 128 // max(S, 128)))  # about the same number of samples whatever the sampler
     ys = torch.linspace(0, H - 1, rows).long().unique()
     idx = (ys[:, None] * W + torch.arange(W)[None]).reshape(-1)
     t0 = time.time()
@@ -260,7 +336,7 @@ def cpu_baseline_frame(args, p, rays, rgb, depth, H, W):
     r = rays[idx.to(rays.device)].cpu()
     torch.set_num_threads(os.cpu_count() if args.cpu_threads <= 0 else args.cpu_threads)
     t0 = time.perf_counter()
-    ret, _ = O.renderer_fn(r, pc, chunk=8192, white_bg=True)
+    ret, _ = O.renderer_fn(r, pc, chunk=8192, white_bg=True, **({} if app_code is None else {"app_code": app_code}))
     dt = time.perf_counter() - t0
     d_rgb = (rgb[idx.to(rgb.device)].cpu() - ret["rgb_map"]).abs().max().item()
     d_dep = (depth[idx.to(rgb.device)].cpu() - ret["depth_map"]).abs().max().item()
@@ -380,7 +456,11 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--streams", type=int, default=2, help="also time the frame with its chunks dealt to this many streams")
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5", "prod"],
+                    help="c4 (default): 1080p frame of the multi-resolution model; prod: the same frame with the reference's "
+                         "production shape (one orientation, AABB sampler, embedding, density projection)")
+    ap.add_argument("--step-ratio", type=float, default=0.5, help="prod: grid cells per sampling step (the reference's default)")
+    ap.add_argument("--no-extra", action="store_true", help="c4: skip the exact-mode and one-orientation timings after the timed region")
     ap.add_argument("--planes", type=int, default=3, help="ndims of the c4 model (3 = XY,XZ,YZ; 1 = XY only)")
     ap.add_argument("--base", type=int, default=1024, help="base plane resolution of c4 (levels x1,x2,x4)")
     ap.add_argument("--height", type=int, default=1080)

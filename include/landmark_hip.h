@@ -268,6 +268,13 @@ int lm_weights(const lm_geom *geom, const float *rays, int64_t N, const uint64_t
                float term_eps, float *w_valid, float *weight_out, uint32_t *app_first, uint32_t *app_cnt,
                uint32_t *app_idx, float *app_w, float *acc, float *depth, uint32_t *counters, void *stream);
 
+/* The colour sum of gridnerf_sequential.py:493-502 / :565-574 over the appearance list lm_weights built:
+ *   rgb_map[r] = clamp(sum_i app_w[first_r + i] * rgb[first_r + i] + (white_bg ? 1 - acc[r] : 0), 0, 1)
+ * with rgb [n_app,3] the colour network's output per list slot (samples outside the list have rgb 0 in
+ * the reference and contribute nothing).  prior art: the volrend kernels of dist_render/kernel/cuda_kernel. */
+int lm_composite_rgb(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w, const float *rgb,
+                     const float *acc, int32_t white_bg, float *rgb_map, void *stream);
+
 /* ---- whole chunk ---------------------------------------------------------------------
  * GridBaseSequential.forward(rays_chunk, white_bg, is_train=False)
  * (gridnerf_sequential.py:439-658) -> rgb_map [N,3], depth_map [N].

@@ -72,6 +72,7 @@ SYMBOLS = {
     "lm_mlp": (C.c_int, [_I32, _P, _I32, _P, _P, _I64, _P, _P]),
     "lm_basis": (C.c_int, [_I32, _P, _I32, _P, _I64, _P, _P]),
     "lm_weights": (C.c_int, [C.POINTER(LmGeom), _P, _I64, _P, _P, _P, _F, _F, _F, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "lm_composite_rgb": (C.c_int, [_I64, _P, _P, _P, _P, _P, _I32, _P, _P]),
     "lm_render_workspace_bytes": (_SZ, [C.POINTER(LmModel), _I64]),
     "lm_app_features": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
     "lm_render": (C.c_int, [C.POINTER(LmModel), _P, _I64, _P, _SZ, _P, _P, _P, _P]),

@@ -229,6 +229,15 @@ int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *ap
     return LM_OK;
 }
 
+extern "C" int lm_composite_rgb(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
+                                const float *rgb, const float *acc, int32_t white_bg, float *rgb_map, void *stream) {
+    LM_REQUIRE(N >= 0, "negative ray count");
+    if (N == 0) return LM_OK;
+    LM_REQUIRE((uint64_t)N < (1ull << 32), "ray count does not fit 32 bits");
+    LM_REQUIRE(app_first && app_cnt && app_w && rgb && acc && rgb_map, "null buffer");
+    return lm_launch_composite(N, app_first, app_cnt, app_w, rgb, acc, white_bg, 0u, rgb_map, (hipStream_t)stream);
+}
+
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
     hipLaunchKernelGGL(k_zero_counters, dim3(1), dim3(64), 0, stream, counters);
     LM_CHECK_LAUNCH("k_zero_counters");

@@ -810,9 +810,14 @@ int launch_app_feat(int nu, const lm_model *m, const PlaneSet &ps, int K, const 
 #define LM_AF_CASE(NU_)                                                                                            \
     case NU_: {                                                                                                    \
         auto kern = &k_app_feat<PREC, T, NU_>;                                                                     \
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                  \
-        if (e != hipSuccess) LM_FAIL(LM_ERR_LAUNCH, "k_app_feat: LDS reservation failed: %s", hipGetErrorString(e)); \
+        static thread_local size_t reserved = 0; /* the attribute is set once per thread, kernel and size */       \
+        if (reserved != lds) {                                                                                     \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
+            if (e != hipSuccess)                                                                                   \
+                LM_FAIL(LM_ERR_LAUNCH, "k_app_feat: LDS reservation failed: %s", hipGetErrorString(e));            \
+            reserved = lds;                                                                                        \
+        }                                                                                                          \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, st, m->geom, ps, K, (const char *)m->mlp_packed, L, rays, \
                            list, count, feat);                                                                     \
         break;                                                                                                     \
@@ -1028,9 +1033,17 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     const PlaneSet ps = make_set(m->density, m->n_planes, &m->geom);
     // as many workgroups as are resident at once (the kernel's register count decides), at most four per CU
     auto resident_grid = [](const void *kernel) {
+        // asked once per thread and kernel: the answer depends on the kernel's registers only
+        static thread_local const void *known[4] = {nullptr, nullptr, nullptr, nullptr};
+        static thread_local unsigned grid[4] = {0, 0, 0, 0};
+        for (int i = 0; i < 4; ++i)
+            if (known[i] == kernel) return grid[i];
         int per_cu = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBlock, 0) != hipSuccess || per_cu < 1) per_cu = 2;
-        return (unsigned)lm_persistent_blocks(std::min(per_cu, 4));
+        const unsigned g = (unsigned)lm_persistent_blocks(std::min(per_cu, 4));
+        for (int i = 0; i < 4; ++i)
+            if (!known[i]) { known[i] = kernel; grid[i] = g; break; }
+        return g;
     };
     int c_max = 0;
     for (int k = 0; k < m->n_planes; ++k) c_max = std::max(c_max, (int)m->density[k].C);

@@ -421,6 +421,10 @@ int lm_check_geom(const lm_geom *g) {
     if (g->div0 != 0 || g->div1 != 0) {
         LM_REQUIRE(g->div0 > 0 && g->div1 > 0 && (int64_t)g->div0 * g->div1 <= 65536, "plane division %d x %d", g->div0,
                    g->div1);
+        // One block: the reference maps block b to the coordinate 2 b / (div0 div1 - 1) - 1 = 0 / 0
+        // (app/models/gridnerf_parallel.py:333-335) and renders NaN; there is nothing to reproduce.
+        if ((int64_t)g->div0 * g->div1 == 1)
+            LM_FAIL(LM_ERR_UNSUPPORTED, "plane division 1 x 1: a single block is the plain (unstacked) layout, set div0 = 0");
         LM_REQUIRE(g->blk_w > 0.0f && g->blk_h > 0.0f, "block size must be positive");
     }
     return LM_OK;

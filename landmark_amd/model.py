@@ -68,7 +68,7 @@ class GridNeRFHIP:
         self.near_far = list(params.near_far)
         self.distance_scale = params.distance_scale
         self.rayMarch_weight_thres = params.rayMarch_weight_thres
-        self.alpha_mask_filter_thre = params.alpha_mask_filter_thre
+        self._alpha_mask_filter_thre = float(params.alpha_mask_filter_thre)
         self.sampling_opt = params.sampling_opt
         self.ndims, self.resMode = params.ndims, list(params.resMode)
         self.nSamples = params.nSamples
@@ -77,6 +77,8 @@ class GridNeRFHIP:
         self.stepSize = params.stepSize
         self._occupancy = occupancy
         self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
+        self._struct_cache: Dict[tuple, L.LmModel] = {}
+        self._need_cache: Dict[tuple, int] = {}
         self._set_alpha_mask(params.alpha_volume, params.alpha_aabb)
         # --- channel-last tables
         self.plane_division = None if params.plane_division is None else [int(v) for v in params.plane_division]
@@ -85,6 +87,10 @@ class GridNeRFHIP:
             if params.ndims != 1:
                 raise L.LandmarkError("a block-stacked model has ndims = 1 (XY planes, z lines)")
             self._n_blocks = self.plane_division[0] * self.plane_division[1]
+            if self._n_blocks == 1:
+                # the reference's block coordinate 2 b / (B - 1) - 1 is 0 / 0 for one block (gridnerf_parallel.py:333-335)
+                raise L.LandmarkError("plane_division [1, 1]: one block is the plain layout; squeeze the block axis "
+                                      "(planes [1,C,h,w], lines [1,C,L,1]) and pass plane_division=None")
         self._tables = []  # keep device tensors alive
         self._density = self._relayout_set(params.density_plane, params.density_line)
         self._app = self._relayout_set(params.app_plane, params.app_line)
@@ -115,10 +121,26 @@ class GridNeRFHIP:
         self._slot_counters = []
         self.counters = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)
 
+    @property
+    def alpha_mask_filter_thre(self) -> float:
+        """Occupancy lookups must exceed this to keep a sample (gridnerf_sequential.py:131, 463)."""
+        return self._alpha_mask_filter_thre
+
+    @alpha_mask_filter_thre.setter
+    def alpha_mask_filter_thre(self, value) -> None:
+        self._alpha_mask_filter_thre = float(value)
+        self._invalidate()  # the cached geometry holds the threshold
+
+    def _invalidate(self) -> None:
+        """Drop everything derived from the geometry (after the occupancy volume or its threshold changed)."""
+        self._geom_cache.clear()
+        self._struct_cache.clear()
+        self._need_cache.clear()
+
     # ------------------------------------------------------------------ construction helpers
     def _set_alpha_mask(self, volume, aabb):
         """Install an occupancy volume [D,H,W] (AlphaGridMask, app/models/alpha_mask.py:16-26) or none."""
-        self._geom_cache.clear()
+        self._invalidate()
         self.alphaMask = None
         self._vol, self._vol_store, self._vol_dtype, self._alpha_aabb = None, None, L.LM_F32, None
         if volume is None:
@@ -256,7 +278,7 @@ class GridNeRFHIP:
             ab = self._alpha_aabb
             g.vol_aabb_min[:] = ab[0].tolist()
             g.vol_inv[:] = (1.0 / (ab[1] - ab[0]) * 2).tolist()
-            g.vol_thre = torch.tensor(p.alpha_mask_filter_thre, dtype=torch.float32).item()
+            g.vol_thre = torch.tensor(self._alpha_mask_filter_thre, dtype=torch.float32).item()
         if self._n_blocks:
             g.div0, g.div1 = self.plane_division
             # the reference divides float tensors by the Python floats 2/div (gridnerf_parallel.py:304-311)
@@ -266,6 +288,17 @@ class GridNeRFHIP:
         return g
 
     def _model_struct(self, S: int, white_bg: bool) -> L.LmModel:
+        """The lm_model of a render with S samples per ray, built once per distinct setting and reused (a caller
+        that keeps small chunks pays for launches only); never carries event handles."""
+        key = (int(S), bool(white_bg), self.mlp_precision, float(self.term_eps), int(self.ray_row_length), id(self._geom_cache))
+        m = self._struct_cache.get(key)
+        if m is None:
+            if len(self._struct_cache) > 64:
+                self._struct_cache.clear()
+            m = self._struct_cache[key] = self._build_model_struct(S, white_bg)
+        return m
+
+    def _build_model_struct(self, S: int, white_bg: bool) -> L.LmModel:
         m = L.LmModel()
         m.geom = self._geom(S)
         m.n_planes = len(self._density)
@@ -293,10 +326,16 @@ class GridNeRFHIP:
         """Device workspace for chunks of up to n_rays rays; grown on demand and reused
         (the role of allocate_tensors, dist_render/kernel/cuda_render_extend.py:35-159).
         Renders that run concurrently on different streams take different slots."""
-        m = self._model_struct(S, True)
-        need = self.lib.lm_render_workspace_bytes(C.byref(m), n_rays)
-        if need == 0:
-            raise L.LandmarkError(self.lib.lm_last_error().decode())
+        key = (int(n_rays), int(S), self.mlp_precision)
+        need = self._need_cache.get(key)
+        if need is None:
+            m = self._model_struct(S, True)
+            need = self.lib.lm_render_workspace_bytes(C.byref(m), n_rays)
+            if need == 0:
+                raise L.LandmarkError(self.lib.lm_last_error().decode())
+            if len(self._need_cache) > 256:
+                self._need_cache.clear()
+            self._need_cache[key] = need
         ws = self._ws.get(slot)
         if ws is None or ws.numel() < need:
             self._ws[slot] = None
@@ -374,6 +413,7 @@ class GridNeRFHIP:
         ws = self.workspace(N, S, slot)
         m = self._model_struct(S, white_bg)
         if events is not None:
+            m = L.LmModel.from_buffer_copy(m)  # the cached struct stays free of event handles
             for i, e in enumerate(events):
                 m.events[i] = e.cuda_event
         cnt = self.slot_counters(slot) if counters is None else counters
@@ -572,6 +612,21 @@ class GridNeRFHIP:
         }
 
     @torch.no_grad()
+    def composite_rgb(self, wres, rgb, white_bg=True):
+        """The per-ray colour sum over the appearance list of a `weights` result; rgb is [n_app,3] in list order."""
+        N = wres["acc_map"].shape[0]
+        rgb = rgb.to(self.device, torch.float32).contiguous()
+        first = wres["app_first"].to(torch.int32).contiguous()
+        cnt = wres["app_cnt"].to(torch.int32).contiguous()
+        out = torch.empty((N, 3), dtype=torch.float32, device=self.device)
+        L.check(
+            self.lib.lm_composite_rgb(N, first.data_ptr(), cnt.data_ptr(), wres["app_w"].contiguous().data_ptr(), rgb.data_ptr(),
+                                      wres["acc_map"].data_ptr(), int(bool(white_bg)), out.data_ptr(), L.current_stream()),
+            "lm_composite_rgb",
+        )
+        return out
+
+    @torch.no_grad()
     def app_features_list(self, cull, wres, precision=None):
         """Fused gather + basis_mat over the appearance list of a `weights` result -> [n_app,27]."""
         old = self.mlp_precision
@@ -589,41 +644,78 @@ class GridNeRFHIP:
         return feat[: wres["n_app"]]
 
 
-def from_reference_model(model, **kw) -> GridNeRFHIP:
-    """Build from an object with the reference model's attributes (a loaded
-    `GridNeRF`, gridnerf_sequential.py:661-747) without importing the reference."""
+def params_from_reference_model(model) -> GridNeRFParams:
+    """The parameter container of an object that carries the reference model's attributes: a loaded `GridNeRF`
+    (gridnerf_sequential.py:46-132, 661-747) or the block-stacked `GridNeRFBranchParallel` a "-merged-stack"
+    checkpoint loads into (planes [1,C,B,h,w], `model.args.plane_division`, gridnerf_parallel.py:299-335).
+    Reads attributes only; the reference is not imported."""
+    args = getattr(model, "args", None)
+
+    def arg(name, default=None):
+        # values the reference keeps on the model where it has them, else in its run arguments
+        # (an ArgsConfig / namespace, or the dict a merged checkpoint stores)
+        if hasattr(model, name):
+            return getattr(model, name)
+        if isinstance(args, dict):
+            return args.get(name, default)
+        return getattr(args, name, default)
+
     lin = [model.renderModule.mlp[i] for i in (0, 2, 4)]
     am = getattr(model, "alphaMask", None)
-    p = GridNeRFParams(
-        aabb=model.aabb.detach().float().cpu(),
-        gridSize=[int(x) for x in model.gridSize.tolist()],
-        density_plane=[t.detach() for t in model.density_plane],
+    planes = [t.detach() for t in model.density_plane]
+    division = None
+    if planes[0].dim() == 5:
+        division = arg("plane_division")
+        if division is None:
+            raise L.LandmarkError("block-stacked planes ([1,C,B,h,w]) but the model's args hold no plane_division")
+        division = [int(v) for v in division]
+    grid = model.gridSize
+    encode_app = bool(arg("encode_app", False))
+    nonlinear = bool(arg("nonlinear_density", False))
+    res_mode = arg("resMode")
+    vol = None
+    if am is not None:
+        vol = am.alpha_volume.detach()
+        vol = vol.reshape(vol.shape[-3:])  # the reference keeps [1,1,D,H,W] (alpha_mask.py:23)
+    return GridNeRFParams(
+        aabb=torch.as_tensor(model.aabb).detach().float().cpu(),
+        gridSize=[int(x) for x in (grid.tolist() if torch.is_tensor(grid) else grid)],
+        density_plane=planes,
         density_line=[t.detach() for t in model.density_line],
         app_plane=[t.detach() for t in model.app_plane],
         app_line=[t.detach() for t in model.app_line],
         basis_mat=model.basis_mat.weight.detach(),
         mlp_w=[l.weight.detach() for l in lin],
         mlp_b=[None if l.bias is None else l.bias.detach() for l in lin],
-        ndims=model.ndims,
-        resMode=list(model.resMode),
+        ndims=int(model.ndims),
+        resMode=[1] if res_mode is None else [int(r) for r in res_mode],
         near_far=[float(x) for x in model.near_far],
         density_shift=float(model.density_shift),
         distance_scale=float(model.distance_scale),
         rayMarch_weight_thres=float(model.rayMarch_weight_thres),
         fea2denseAct=model.fea2denseAct,
         step_ratio=float(model.step_ratio),
-        sampling_opt=int(model.sampling_opt),
-        n_importance=int(model.n_importance),
-        view_pe=model.view_pe,
-        fea_pe=model.fea_pe,
-        app_dim=model.app_dim,
-        featureC=model.featureC,
-        alpha_volume=None if am is None else am.alpha_volume[0, 0].detach(),
-        alpha_aabb=None if am is None else am.aabb.detach().cpu(),
-        alpha_mask_filter_thre=float(model.alpha_mask_filter_thre),
-        encode_app=bool(getattr(model.args, "encode_app", False)),
-        embedding_app=model.embedding_app.weight.detach() if getattr(model.args, "encode_app", False) else None,
-        nonlinear_density=bool(getattr(model, "nonlinear_density", False)),
-        basis_den=model.basis_den.weight.detach() if getattr(model, "nonlinear_density", False) else None,
+        sampling_opt=int(arg("sampling_opt", 0)),
+        n_importance=int(arg("n_importance", 128)),
+        view_pe=int(model.view_pe),
+        fea_pe=int(model.fea_pe),
+        app_dim=int(model.app_dim),
+        featureC=int(model.featureC),
+        alpha_volume=vol,
+        alpha_aabb=None if am is None else torch.as_tensor(am.aabb).detach().float().cpu(),
+        alpha_mask_filter_thre=float(arg("alpha_mask_filter_thre", 0.0)),
+        alphaMask_thres=float(arg("alphaMask_thres", 0.001)),
+        encode_app=encode_app,
+        embedding_app=model.embedding_app.weight.detach() if encode_app else None,
+        nonlinear_density=nonlinear,
+        basis_den=model.basis_den.weight.detach() if nonlinear else None,
+        plane_division=division,
     )
-    return GridNeRFHIP(p, **kw)
+
+
+def from_reference_model(model, **kw) -> GridNeRFHIP:
+    """Wrap an object with the reference model's attributes (see params_from_reference_model);
+    keyword arguments go to GridNeRFHIP (device, mlp_precision, term_eps, ...)."""
+    if isinstance(model, GridNeRFHIP):
+        return model
+    return GridNeRFHIP(params_from_reference_model(model), **kw)

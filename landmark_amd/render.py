@@ -44,13 +44,21 @@ class MultiBlockParallelHIP:
     """Pre-sized workspace + forward, the calling convention dist_render's inferer installs
     with set_forward_func (dist_render/ddp_infer/inferer_impl.py:351-366)."""
 
-    def __init__(self):
+    def __init__(self, **model_kw):
+        """Keyword arguments (device, mlp_precision, term_eps, ...) are used when allocate_tensors has to
+        wrap a reference model itself."""
         self._tensorf = None
+        self._model_kw = model_kw
 
     def allocate_tensors(self, tensorf, N_rays):
-        self._tensorf = tensorf
-        S = tensorf._samples_for(-1)
-        tensorf.workspace(int(N_rays), S)
+        """`tensorf` is what dist_render's inferer passes: its loaded reference model, single or block-stacked
+        (inferer_impl.py:354-362), which is wrapped here; an already wrapped GridNeRFHIP is taken as it is."""
+        from .model import from_reference_model
+
+        self._tensorf = from_reference_model(tensorf, **self._model_kw)
+        S = self._tensorf._samples_for(-1)
+        self._tensorf.workspace(int(N_rays), S)
+        return self._tensorf
 
     def forward(self, rays_chunk, app_code=None, white_bg=True):
         if self._tensorf is None:

@@ -241,9 +241,11 @@ def c1_rays(H=400, W=400, seed=0, device="cpu") -> torch.Tensor:
     return pinhole_rays(H, W, focal, sphere_pose(2.5, seed), device=device)
 
 
-def c4_scene(P: int = 3, base: int = 1024, device="cuda", density_shift: float = 0.0, alpha_dims=(256, 256, 256)):
+def c4_scene(P: int = 3, base: int = 1024, device="cuda", density_shift: float = 0.0, alpha_dims=(256, 256, 256), **kw):
     """Full-frame multi-resolution model: levels base, 2*base, 4*base; 16 + 48 ch fp32,
     N(0, 0.1); occupancy from 64 seeded Gaussian blobs at about 30 %."""
+    cfg = dict(sampling_opt=1, n_importance=128)
+    cfg.update(kw)
     p = make_params(
         seed=4,
         gridSize=(base, base, base),
@@ -252,8 +254,7 @@ def c4_scene(P: int = 3, base: int = 1024, device="cuda", density_shift: float =
         device=device,
         near_far=[0.5, 6.0],
         density_shift=density_shift,
-        sampling_opt=1,
-        n_importance=128,
+        **cfg,
     )
     p.alpha_volume = blob_occupancy(alpha_dims, 64, 0.30, seed=4, device=device)
     p.alpha_aabb = p.aabb.clone()
@@ -264,6 +265,18 @@ def c4_scene(P: int = 3, base: int = 1024, device="cuda", density_shift: float =
 def c4_rays(H=1080, W=1920, frame=0, device="cuda") -> torch.Tensor:
     focal = 1483.6378 * (W / 1920.0)  # dist_render/ddp_infer/nerf_inferer.py:404
     return pinhole_rays(H, W, focal, orbit_pose(2.6, 1.9, frame), device=device)
+
+
+def production_scene(base: int = 1024, step_ratio: float = 0.5, device="cuda", density_shift: float = 0.0):
+    """The shape most of the reference's run configurations use (confs/*.txt): one plane orientation
+    (ndims 1) at three levels, the equal-step AABB sampler (sampling_opt 0) with step_ratio grid cells per
+    step (app/tools/config_parser.py:153-155: 0.5, i.e. several thousand samples per ray, nearly all of them
+    culled by the occupancy volume), the appearance embedding, the density projection and biases in the
+    colour network.  Tables, occupancy volume and camera are those of the full-frame multi-resolution scene."""
+    p = c4_scene(P=1, base=base, device=device, density_shift=density_shift, sampling_opt=0, step_ratio=step_ratio,
+                 encode_app=True, nonlinear_density=True)
+    p.basis_den = p.basis_den.abs()  # keep relu(basis_den(.)) from zeroing half of the volume
+    return p
 
 
 def c5_scene(res: int = 8192, device="cuda", density_shift: float = 0.0):

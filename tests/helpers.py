@@ -62,3 +62,56 @@ def load_golden(name, kind="forward"):
         plane_division=cfg.get("plane_division"),
     )
     return p, data, cfg
+
+
+def reference_model_stub(p: GridNeRFParams, args_as_dict=False):
+    """An object carrying exactly the attributes a loaded reference model has (GridBaseSequential.__init__ and
+    GridNeRF.init_svd_volume, app/models/gridnerf_sequential.py:46-132, 669-683; AlphaGridMask,
+    app/models/alpha_mask.py:16-26; MLPRender_Fea.mlp, app/models/mlp_render_fea.py:30-41): module containers
+    for the networks, tensors for the tables, the run's arguments under `.args`.  The reference itself is
+    not imported."""
+    from types import SimpleNamespace
+
+    import torch.nn as nn
+
+    def linear(w, b):
+        lin = nn.Linear(w.shape[1], w.shape[0], bias=b is not None)
+        with torch.no_grad():
+            lin.weight.copy_(w)
+            if b is not None:
+                lin.bias.copy_(b)
+        return lin
+
+    mlp = nn.Sequential(linear(p.mlp_w[0], p.mlp_b[0]), nn.ReLU(inplace=True), linear(p.mlp_w[1], p.mlp_b[1]),
+                        nn.ReLU(inplace=True), linear(p.mlp_w[2], p.mlp_b[2]))
+    args = dict(
+        distributed=False, run_nerf=False, nonlinear_density=p.nonlinear_density, ndims=p.ndims, resMode=list(p.resMode),
+        sampling_opt=p.sampling_opt, bias_enable=int(p.mlp_b[0] is not None), encode_app=p.encode_app,
+        n_importance=p.n_importance, alpha_mask_filter_thre=p.alpha_mask_filter_thre, ckpt=None, device="cpu",
+    )
+    if p.plane_division is not None:
+        args["plane_division"] = list(p.plane_division)
+    m = SimpleNamespace(
+        aabb=p.aabb.clone(), gridSize=torch.tensor(p.gridSize), device="cpu",
+        density_plane=nn.ParameterList([nn.Parameter(t.clone()) for t in p.density_plane]),
+        density_line=nn.ParameterList([nn.Parameter(t.clone()) for t in p.density_line]),
+        app_plane=nn.ParameterList([nn.Parameter(t.clone()) for t in p.app_plane]),
+        app_line=nn.ParameterList([nn.Parameter(t.clone()) for t in p.app_line]),
+        basis_mat=linear(p.basis_mat, None), renderModule=SimpleNamespace(mlp=mlp),
+        ndims=p.ndims, resMode=list(p.resMode), near_far=list(p.near_far), density_shift=p.density_shift,
+        distance_scale=p.distance_scale, rayMarch_weight_thres=p.rayMarch_weight_thres, fea2denseAct=p.fea2denseAct,
+        step_ratio=p.step_ratio, sampling_opt=p.sampling_opt, n_importance=p.n_importance, view_pe=p.view_pe, fea_pe=p.fea_pe,
+        pos_pe=6, app_dim=p.app_dim, featureC=p.featureC, alpha_mask_filter_thre=p.alpha_mask_filter_thre,
+        alphaMask_thres=p.alphaMask_thres, nonlinear_density=p.nonlinear_density, run_nerf=False, alphaMask=None,
+        args=args if args_as_dict else SimpleNamespace(**args),
+    )
+    if p.alpha_volume is not None:
+        m.alphaMask = SimpleNamespace(alpha_volume=p.alpha_volume.clone().view(1, 1, *p.alpha_volume.shape[-3:]),
+                                      aabb=p.alpha_aabb.clone(), device="cpu")
+    if p.nonlinear_density:
+        m.basis_den = linear(p.basis_den, None)
+    if p.encode_app:
+        m.embedding_app = nn.Embedding(p.embedding_app.shape[0], p.embedding_app.shape[1])
+        with torch.no_grad():
+            m.embedding_app.weight.copy_(p.embedding_app)
+    return m

@@ -305,6 +305,36 @@ def test_weights_against_raw2alpha(gpu_lib):
         assert torch.equal(seg, w["app_mask"][r].nonzero()[:, 0] + r * S)
 
 
+@pytest.mark.parametrize("white_bg", [True, False])
+def test_colour_sum_stage(gpu_lib, white_bg):
+    """lm_composite_rgb alone: per-ray sum of weight * rgb over the appearance list, white background before the
+    clamp, against the dense tensor expression of the reference (rgb zero outside the mask)."""
+    p = _scene(S=128, thre=0.0)
+    rays = scenes.pinhole_rays(64, 64, 60.0, scenes.sphere_pose(2.5, 5))
+    m = _model(p)
+    cull = m.sample_cull(rays)
+    w = m.weights(cull, m.density_valid(cull))
+    assert w["n_app"] > 1000
+    g = torch.Generator(device="cuda").manual_seed(3)
+    rgb = torch.rand((w["n_app"], 3), device="cuda", generator=g) * 1.6 - 0.2  # sums that reach past both clamp limits
+    got = m.composite_rgb(w, rgb, white_bg=white_bg)
+    N, S = rays.shape[0], cull["S"]
+    dense = torch.zeros((N * S, 3), device="cuda", dtype=torch.float64)
+    dense[w["app_idx"]] = rgb.double()
+    exp = (w["weight"].double()[..., None] * dense.view(N, S, 3)).sum(1)
+    if white_bg:
+        exp = exp + (1.0 - w["acc_map"].double()[:, None])
+    exp = exp.clamp(0, 1)
+    assert (got.double() - exp).abs().max().item() <= 2e-6
+    assert bool((got == 0).any()) or bool((got == 1).any())  # the clamp was reached
+    empty = w["app_cnt"] == 0
+    assert bool(empty.any())
+    if white_bg:
+        assert torch.equal(got[empty], (1.0 - w["acc_map"][empty])[:, None].expand(-1, 3).clamp(0, 1))
+    else:
+        assert bool((got[empty] == 0).all())
+
+
 @pytest.mark.parametrize("prec,tol", [("f32", 5e-6), ("f16x2", 5e-6), ("f16", 5e-3), ("bf16", 4e-2)])
 def test_fused_appearance_features(gpu_lib, prec, tol):
     """gather + basis_mat over the appearance list against the oracle's compute_appfeature"""
@@ -642,6 +672,28 @@ def test_stacked_model_random_scene(gpu_lib, div, res, prec):
     assert (out["rgb_map"].cpu() - ref["rgb_map"])[~band].abs().max().item() <= RGB_TOL_F32
     assert (out["depth_map"].cpu() - ref["depth_map"])[~band].abs().max().item() <= RGB_TOL_F32
     assert int(band.sum()) <= max(2, rays.shape[0] // 500)
+
+
+def test_stacked_model_single_block_is_refused(gpu_lib):
+    """plane_division (1, 1): the reference's block coordinate is 0 / 0 there (its render is NaN, and so is the
+    oracle's); the wrapper and the C ABI refuse it instead of inventing a result."""
+    from landmark_amd import _lib as L
+
+    p = scenes.make_params(seed=11, gridSize=(10, 9, 12), near_far=[0.5, 4.5], n_importance=32, sampling_opt=1,
+                           density_shift=0.0, ndims=1, plane_division=(1, 1))
+    rays = scenes.pinhole_rays(8, 8, 7.0, scenes.sphere_pose(2.5, 7))
+    assert torch.isnan(O.render_chunk(p, rays)["rgb_map"]).any()
+    with pytest.raises(L.LandmarkError, match="one block"):
+        _model(p)
+    p2 = scenes.make_params(seed=11, gridSize=(10, 9, 12), near_far=[0.5, 4.5], n_importance=32, sampling_opt=1,
+                            density_shift=0.0, ndims=1, plane_division=(2, 1))
+    m = _model(p2)
+    g = m._geom(32)
+    g.div0 = g.div1 = 1
+    cnt = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device="cuda")
+    rc = m.lib.lm_sample_cull(C.byref(g), rays.cuda().data_ptr(), rays.shape[0], cnt.data_ptr(), cnt.data_ptr(), None,
+                              cnt.data_ptr(), None, cnt.data_ptr(), L.current_stream())
+    assert rc == -2 and b"1 x 1" in m.lib.lm_last_error()
 
 
 @pytest.mark.parametrize("div", [(2, 3), (5, 4), (7, 1)])
