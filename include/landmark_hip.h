@@ -286,6 +286,21 @@ size_t lm_render_workspace_bytes(const lm_model *model, int64_t N);
 int lm_render(const lm_model *model, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
               float *rgb_map, float *depth_map, uint32_t *counters, void *stream);
 
+/* lm_render out of a workspace built into the library, for callers that cannot allocate device
+ * memory or pass a workspace along: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference (its fused path allocates its buffers
+ * with torch, dist_render/kernel/cuda_render_extend.py:35-159).  Same arguments, results and
+ * stages as lm_render; the workspace is a LM_STATIC_WORKSPACE_BYTES array in the library's device
+ * image (every GPU the library runs on holds one until the process ends).  The call allocates
+ * nothing; the array's address is looked up on the first call on a device.  A chunk whose
+ * lm_render_workspace_bytes() exceeds the array is refused with LM_ERR_WORKSPACE (80 MiB holds
+ * 4096 rays of 128 samples).  All calls on one GPU share the array: calls that overlap on one
+ * GPU (different streams or threads) race; everything that must start at zero is cleared by the
+ * call's own kernels on `stream`. */
+#define LM_STATIC_WORKSPACE_BYTES (80u << 20)
+int lm_render_static(const lm_model *model, const float *rays, int64_t N, float *rgb_map, float *depth_map,
+                     uint32_t *counters, void *stream);
+
 /* ---- either side of the path in the serving loop ------------------------------------------
  * lm_generate_rays: rays[j*W+i] = (pose[:,3], pose[:,:3] @ (dir_x[i], dir_y[j], -1)), the
  * pinhole rays of dist_render/dataset/utils.py:57-113 (generate_rays).  dir_x [W] and dir_y [H]

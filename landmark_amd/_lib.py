@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(HERE, "liblandmark_hip.so")
 
 LM_MAX_PLANES = 12
+LM_STATIC_WORKSPACE_BYTES = 80 << 20
 LM_N_STAGES = 6
 STAGE_NAMES = ["cull", "density_march", "app_list", "app_gather", "colour", "composite"]
 LM_ABI_VERSION = 2  # include/landmark_hip.h
@@ -76,6 +77,7 @@ SYMBOLS = {
     "lm_render_workspace_bytes": (_SZ, [C.POINTER(LmModel), _I64]),
     "lm_app_features": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),
     "lm_render": (C.c_int, [C.POINTER(LmModel), _P, _I64, _P, _SZ, _P, _P, _P, _P]),
+    "lm_render_static": (C.c_int, [C.POINTER(LmModel), _P, _I64, _P, _P, _P, _P]),
     "lm_generate_rays": (C.c_int, [_P, _P, _P, _I32, _I32, _P, _P]),
     "lm_rgba8": (C.c_int, [_P, _I64, _P, _P]),
     "lm_density_valid": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _P, _P]),

@@ -2,6 +2,7 @@
 #include <stdarg.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "lm_common.h"
 
@@ -161,6 +162,9 @@ int check_model(const lm_model *m, int *K) {
         }
     return LM_OK;
 }
+
+int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
+                 float *rgb_map, float *depth_map, uint32_t *counters, void *stream);
 }  // namespace
 
 extern "C" size_t lm_render_workspace_bytes(const lm_model *m, int64_t N) {
@@ -173,6 +177,58 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
                          float *rgb_map, float *depth_map, uint32_t *counters, void *stream) {
     int K;
     if (int rc = check_model(m, &K)) return rc;
+    return render_chunk(m, K, rays, N, workspace, workspace_bytes, rgb_map, depth_map, counters, stream);
+}
+
+// ---- the same render out of a workspace that lives in the library's own image ------------------
+// One array per GPU (each device that loads the code object holds its own copy at its own
+// address).  In host code the array's name is only a handle for hipGetSymbolAddress: the device
+// address is looked up once per device and everything after that uses the pointer.
+static __device__ __align__(256) unsigned char scratch[LM_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_workspace(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        LM_FAIL(LM_ERR_LAUNCH, "lm_render_static: no current device (or device index %d beyond %d)", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            LM_FAIL(LM_ERR_LAUNCH, "lm_render_static: address of the built-in workspace on device %d: %s", dev,
+                    hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return LM_OK;
+}
+}  // namespace
+
+extern "C" int lm_render_static(const lm_model *m, const float *rays, int64_t N, float *rgb_map, float *depth_map,
+                                uint32_t *counters, void *stream) {
+    int K;
+    if (int rc = check_model(m, &K)) return rc;
+    LM_REQUIRE(N >= 0, "negative ray count");
+    if (N == 0) return LM_OK;
+    const size_t need = carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m), m->weight_thres).total;
+    if (need > (size_t)LM_STATIC_WORKSPACE_BYTES)
+        LM_FAIL(LM_ERR_WORKSPACE,
+                "lm_render_static: %lld rays x %d samples need %zu bytes of workspace, the built-in one has %zu; "
+                "render fewer rays per call or use lm_render with a workspace of your own",
+                (long long)N, m->geom.S, need, (size_t)LM_STATIC_WORKSPACE_BYTES);
+    void *ws = nullptr;
+    if (int rc = static_workspace(&ws)) return rc;
+    return render_chunk(m, K, rays, N, ws, (size_t)LM_STATIC_WORKSPACE_BYTES, rgb_map, depth_map, counters, stream);
+}
+
+namespace {
+int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
+                 float *rgb_map, float *depth_map, uint32_t *counters, void *stream) {
     LM_REQUIRE(N >= 0, "negative ray count");
     if (N == 0) return LM_OK;
     LM_REQUIRE(rays && rgb_map && depth_map, "null buffer");
@@ -220,3 +276,4 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
     mark(LM_STAGE_COMPOSITE);
     return LM_OK;
 }
+}  // namespace

@@ -1,0 +1,91 @@
+"""lm_render_static: the whole-chunk render out of the workspace built into the library.
+
+Called through the C ABI and compared with lm_render (caller-owned workspace) on the same
+inputs: same kernels, same stage order, so rgb, depth and the sample counters must be equal
+bit for bit.  Two calls in a row share the built-in array, the second with fewer rays (what
+the first left behind must not leak into it), then a larger one again.  Oversized chunks are
+refused with a status code."""
+import ctypes as C
+
+import pytest
+import torch
+
+from landmark_amd import _lib as L
+from landmark_amd import scenes
+from oracle import gridnerf_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _scene(S, opt, seed=11):
+    p = scenes.make_params(seed=seed, gridSize=(9, 11, 13), near_far=[0.5, 4.5], n_importance=S, sampling_opt=opt,
+                           density_shift=0.0, step_ratio=0.3, resMode=(1, 2))
+    for t in p.density_plane:
+        t.mul_(6.0)
+    p.alpha_volume = scenes.blob_occupancy((13, 11, 9), 6, 0.45, seed=seed)
+    p.alpha_aabb = p.aabb.clone()
+    return p
+
+
+def _both(model, rays, S, white_bg=True):
+    """(rgb, depth, counters) from lm_render and from lm_render_static."""
+    lib, dev = model.lib, model.device
+    N = rays.shape[0]
+    m = model._model_struct(S, white_bg)
+    out = []
+    for static in (False, True):
+        rgb = torch.full((N, 3), -1.0, device=dev)
+        depth = torch.full((N,), -1.0, device=dev)
+        cnt = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=dev)
+        if static:
+            rc = lib.lm_render_static(C.byref(m), rays.data_ptr(), N, rgb.data_ptr(), depth.data_ptr(), cnt.data_ptr(),
+                                      L.current_stream())
+        else:
+            ws = model.workspace(N, S)
+            rc = lib.lm_render(C.byref(m), rays.data_ptr(), N, ws.data_ptr(), ws.numel(), rgb.data_ptr(), depth.data_ptr(),
+                               cnt.data_ptr(), L.current_stream())
+        L.check(rc, "lm_render_static" if static else "lm_render")
+        torch.cuda.synchronize()
+        out.append((rgb, depth, cnt[:3].clone()))
+    return out
+
+
+@pytest.mark.parametrize("opt,S", [(1, 128), (0, 100)])
+def test_static_workspace_render_equals_lm_render(gpu_lib, opt, S):
+    from landmark_amd.model import GridNeRFHIP
+
+    p = _scene(S, opt)
+    model = GridNeRFHIP(p, mlp_precision="f16x2")
+    big = scenes.pinhole_rays(60, 50, 52.0, scenes.sphere_pose(2.5, 9)).cuda()  # 3000 rays
+    small = big[1234:1234 + 517].contiguous()
+    for rays in (big, small, big):  # the second call is smaller than the first and finds its leftovers
+        (rgb_a, dep_a, cnt_a), (rgb_b, dep_b, cnt_b) = _both(model, rays, S)
+        assert int(cnt_a[L.LM_STAT_N_APP]) > 0, "scene must exercise the colour network"
+        assert torch.equal(cnt_a, cnt_b)
+        assert torch.equal(rgb_a, rgb_b) and torch.equal(dep_a, dep_b)
+        assert float(rgb_b.min()) >= 0.0 and float(rgb_b.max()) <= 1.0
+    # and both agree with the oracle on the small call
+    ref = O.render_chunk(p, small.cpu(), N_samples=S, return_aux=True)
+    band = ((ref["weight"] - 1e-3).abs() < 2e-7).any(-1)
+    (_, _, _), (rgb_s, dep_s, _) = _both(model, small, S)
+    assert (rgb_s.cpu() - ref["rgb_map"]).abs().max(-1).values[~band].max().item() <= 1e-4
+    assert (dep_s.cpu() - ref["depth_map"]).abs()[~band].max().item() <= 1e-4
+
+
+def test_static_workspace_refuses_oversized_chunks(gpu_lib):
+    from landmark_amd.model import GridNeRFHIP
+
+    p = _scene(128, 1)
+    model = GridNeRFHIP(p)
+    lib = model.lib
+    m = model._model_struct(128, True)
+    N = 1 << 16  # 65536 rays x 128 samples: far beyond the built-in array
+    assert lib.lm_render_workspace_bytes(C.byref(m), N) > L.LM_STATIC_WORKSPACE_BYTES
+    rays = torch.zeros((N, 6), device="cuda")
+    rgb = torch.zeros((N, 3), device="cuda")
+    depth = torch.zeros((N,), device="cuda")
+    rc = lib.lm_render_static(C.byref(m), rays.data_ptr(), N, rgb.data_ptr(), depth.data_ptr(), None, L.current_stream())
+    assert rc == -4 and b"built-in" in lib.lm_last_error()
+    # the largest chunk lm_render_workspace_bytes admits is accepted (4096 rays of 128 samples fit)
+    assert lib.lm_render_workspace_bytes(C.byref(m), 4096) <= L.LM_STATIC_WORKSPACE_BYTES
+    assert lib.lm_render_static(C.byref(m), rays.data_ptr(), 0, rgb.data_ptr(), depth.data_ptr(), None, L.current_stream()) == 0
