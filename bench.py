@@ -148,7 +148,18 @@ def bench_frame(args, workload):
     rgb = torch.empty((N, 3), device=dev)
     depth = torch.empty((N,), device=dev)
     counters = torch.zeros((n_chunks, L.LM_STAT_WORDS), dtype=torch.int32, device=dev)
+    # one untimed frame sizes the workspace: the library starts from a guess of the samples per ray, reads the
+    # counters and repeats chunks that did not fit (GridNeRFHIP.finish_chunks); the timed frames then run on a
+    # workspace of fixed size, and the overflow counter is checked again after them
+    done = []
+    for ci in range(n_chunks):
+        sl = slice(ci * chunk, min((ci + 1) * chunk, N))
+        model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci])
+        done.append((sl, counters[ci]))
+    repeats = model.finish_chunks(done, rays, rgb, depth, white_bg=True)
     ws = model.workspace(chunk, S)
+    log(f"[bench] workspace {ws.numel() / 1e9:.2f} GB for chunks of {chunk} rays ({repeats} chunk renders repeated while sizing it; "
+        f"samples per ray it holds: valid {model.samples_per_ray[0]:.1f}, appearance {model.samples_per_ray[1]:.1f})")
     n_ev = L.LM_N_STAGES + 1
     events = [[[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(n_chunks)] for _ in range(args.steps)]
     for per_step in events:
@@ -219,7 +230,7 @@ def bench_frame(args, workload):
     cnt = counters.cpu().long() & 0xFFFFFFFF
     n_valid, n_app = int(cnt[:, L.LM_STAT_N_VALID].sum()), int(cnt[:, L.LM_STAT_N_APP].sum())
     n_marched = int(cnt[:, L.LM_STAT_N_MARCHED].sum())
-    overflow = int(cnt[:, L.LM_STAT_OVERFLOW].sum()) if hasattr(L, "LM_STAT_OVERFLOW") else 0
+    overflow = int(cnt[:, L.LM_STAT_OVERFLOW].sum())
     if overflow:
         raise RuntimeError(f"{overflow} rays did not fit the workspace capacity: the timed frames are incomplete")
     stage_ms = [0.0] * L.LM_N_STAGES  # per frame, averaged over steps

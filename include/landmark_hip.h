@@ -29,8 +29,9 @@
 extern "C" {
 #endif
 
-/* Changes whenever a struct, an enum value or the meaning of an argument does (2: 16-word counter block). */
-#define LM_ABI_VERSION 2
+/* Changes whenever a struct, an enum value or the meaning of an argument does (2: 16-word counter block;
+ * 3: workspace capacities in lm_model, LM_STAT_OVERFLOW). */
+#define LM_ABI_VERSION 3
 #define LM_MAX_PLANES 12 /* ndims * len(resMode) */
 
 typedef enum lm_status {
@@ -140,6 +141,16 @@ typedef struct lm_model {
      * multiple of 8: rays are visited in the order given. */
     int32_t ray_row;
     int32_t reserved_;
+    /* Workspace capacities of one lm_render call, in samples: room for the chunk's valid samples and for its
+     * appearance samples (weight > weight_thres).  0 = the worst case (every sample valid, every ray with
+     * min(S, 1 / weight_thres) appearance samples), which cannot overflow; the reference's fused path sizes its
+     * buffers for 64 rows per ray instead (dist_render/kernel/cuda_render_extend.py:35-159).  A ray whose samples
+     * do not fit is rendered as if it had none and counted in counters[LM_STAT_OVERFLOW]: the caller reads the
+     * counters, and when that word is not zero repeats the call with capacities of at least
+     * counters[LM_STAT_N_VALID] and counters[LM_STAT_N_APP] (both keep counting past the capacity; after a
+     * valid-sample overflow N_APP is a lower bound and the repeat may report a second, appearance overflow). */
+    int64_t cap_valid;
+    int64_t cap_app;
     /* Optional timing hooks: hipEvent_t handles created by the caller, or NULL.  lm_render
      * records events[0] before its first kernel and events[i] after stage i on `stream`
      * (LM_STAGE_*); it never waits on them. */
@@ -152,7 +163,9 @@ typedef struct lm_model {
  * marching queue hands out the long rays first; QUEUE..QUEUE+7: internal cursors of that queue,
  * one per XCD.  Two lm_render calls that may run at the same time (different streams) need a
  * counter block and a workspace each. */
-enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_MARCHED = 2, LM_STAT_BINS = 4, LM_STAT_QUEUE = 8, LM_STAT_WORDS = 16 };
+/* OVERFLOW: rays dropped because their samples did not fit lm_model.cap_valid / cap_app (0 unless capacities
+ * below the worst case were asked for). */
+enum { LM_STAT_N_VALID = 0, LM_STAT_N_APP = 1, LM_STAT_N_MARCHED = 2, LM_STAT_OVERFLOW = 3, LM_STAT_BINS = 4, LM_STAT_QUEUE = 8, LM_STAT_WORDS = 16 };
 
 int lm_abi_version(void);
 const char *lm_last_error(void);

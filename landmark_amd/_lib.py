@@ -15,8 +15,8 @@ LM_MAX_PLANES = 12
 LM_STATIC_WORKSPACE_BYTES = 80 << 20
 LM_N_STAGES = 6
 STAGE_NAMES = ["cull", "density_march", "app_list", "app_gather", "colour", "composite"]
-LM_ABI_VERSION = 2  # include/landmark_hip.h
-LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_N_MARCHED, LM_STAT_BINS, LM_STAT_QUEUE, LM_STAT_WORDS = 0, 1, 2, 4, 8, 16
+LM_ABI_VERSION = 3  # include/landmark_hip.h
+LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_N_MARCHED, LM_STAT_OVERFLOW, LM_STAT_BINS, LM_STAT_QUEUE, LM_STAT_WORDS = 0, 1, 2, 3, 4, 8, 16
 LM_F32, LM_F16, LM_U8, LM_CELLS = 0, 1, 2, 3
 LM_SAMPLER_AABB, LM_SAMPLER_HULL = 0, 1
 LM_ACT_SOFTPLUS, LM_ACT_RELU = 0, 1
@@ -48,7 +48,7 @@ class LmModel(C.Structure):
         ("density", LmPlane * LM_MAX_PLANES), ("app", LmPlane * LM_MAX_PLANES),
         ("density_basis", C.c_void_p), ("act", C.c_int32), ("density_shift", C.c_float), ("distance_scale", C.c_float), ("weight_thres", C.c_float),
         ("mlp_prec", C.c_int32), ("mlp_packed", C.c_void_p), ("white_bg", C.c_int32), ("term_eps", C.c_float),
-        ("ray_row", C.c_int32), ("reserved_", C.c_int32),
+        ("ray_row", C.c_int32), ("reserved_", C.c_int32), ("cap_valid", C.c_int64), ("cap_app", C.c_int64),
         ("events", C.c_void_p * (LM_N_STAGES + 1)),
     ]
 

@@ -77,22 +77,28 @@ int lm_check_geom(const lm_geom *g);
 int lm_check_planes(const lm_plane *planes, int32_t n, int *dtype_out, int *K_out);
 int lm_app_feat_supported(const lm_model *m);
 int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *feat, const float *rays,
-                         const uint32_t *app_idx, const uint32_t *count, float *rgb, hipStream_t stream);
+                         const uint32_t *app_idx, const uint32_t *count, uint32_t cap, float *rgb, hipStream_t stream);
+int lm_launch_app_features(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *count, uint32_t cap,
+                           float *feat, hipStream_t st);
+int lm_launch_app_products(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *count, uint32_t cap,
+                           float *products, hipStream_t st);
 int lm_launch_composite(int64_t N, const uint32_t *app_first, const uint32_t *app_cnt, const float *app_w,
                         const float *rgb, const float *acc, int white_bg, uint32_t row, float *rgb_map,
                         hipStream_t stream);
 int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
-                         uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st);
+                         uint32_t *app_cnt, uint32_t *p_end, uint32_t row, uint32_t cap_valid, uint32_t *overflow,
+                         hipStream_t st);
 int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
-                        float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
-                        uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, hipStream_t stream);
+                        float weight_thres, uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
+                        uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, uint32_t cap_app,
+                        uint32_t *overflow, hipStream_t stream);
 int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
                     const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid, float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st);
 int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
-                    float *feat, hipStream_t st);
+                    uint32_t cap, float *feat, hipStream_t st);
 
 namespace {
 struct Workspace {
@@ -110,10 +116,12 @@ struct Workspace {
     float *products;  // only when the fused appearance gather does not cover the model
     float *acc;
     uint32_t *counters;
+    uint64_t cap_valid, cap_app;  // room for valid samples and for appearance samples
     size_t total;
 };
 
-Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products, float weight_thres) {
+Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products, float weight_thres, int64_t want_valid,
+                int64_t want_app) {
     Workspace w;
     size_t o = 0;
     auto take = [&](size_t bytes) {
@@ -126,9 +134,12 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products,
     // reference's cumulative-product guard), so at most 1 / threshold of them exceed the threshold.
     uint64_t per_ray = (uint64_t)S;
     if (weight_thres > 0.0f) per_ray = std::min<uint64_t>(per_ray, (uint64_t)(1.001 / (double)weight_thres) + 2);
-    const uint64_t cap = (uint64_t)N * per_ray;
+    // capacities below the worst case are the caller's choice (lm_model.cap_valid / cap_app); kernels check them
+    const uint64_t cap = want_app > 0 ? std::min<uint64_t>((uint64_t)want_app, (uint64_t)N * per_ray) : (uint64_t)N * per_ray;
+    w.cap_app = cap;
+    w.cap_valid = want_valid > 0 ? std::min<uint64_t>((uint64_t)want_valid, total) : total;
     w.bitmap = (uint64_t *)take(n_words * 8);
-    w.w_valid = (float *)take(total * 4);
+    w.w_valid = (float *)take(w.cap_valid * 4);
     w.app_first = (uint32_t *)take((uint64_t)N * 4);
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
     w.p_first = (uint32_t *)take((uint64_t)N * 4);
@@ -170,7 +181,8 @@ int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *w
 extern "C" size_t lm_render_workspace_bytes(const lm_model *m, int64_t N) {
     int K;
     if (check_model(m, &K) || N <= 0) return 0;
-    return carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m), m->weight_thres).total;
+    if (m->cap_valid < 0 || m->cap_app < 0) return 0;
+    return carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m), m->weight_thres, m->cap_valid, m->cap_app).total;
 }
 
 extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *workspace, size_t workspace_bytes,
@@ -215,7 +227,8 @@ extern "C" int lm_render_static(const lm_model *m, const float *rays, int64_t N,
     if (int rc = check_model(m, &K)) return rc;
     LM_REQUIRE(N >= 0, "negative ray count");
     if (N == 0) return LM_OK;
-    const size_t need = carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m), m->weight_thres).total;
+    LM_REQUIRE(m->cap_valid >= 0 && m->cap_app >= 0, "negative workspace capacity");
+    const size_t need = carve(nullptr, N, m->geom.S, K, !lm_app_feat_supported(m), m->weight_thres, m->cap_valid, m->cap_app).total;
     if (need > (size_t)LM_STATIC_WORKSPACE_BYTES)
         LM_FAIL(LM_ERR_WORKSPACE,
                 "lm_render_static: %lld rays x %d samples need %zu bytes of workspace, the built-in one has %zu; "
@@ -236,7 +249,8 @@ int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *w
     const int S = m->geom.S;
     LM_REQUIRE((uint64_t)N * (uint64_t)S < (1ull << 32), "N*S does not fit 32-bit sample indices; split the chunk");
     const bool fused = lm_app_feat_supported(m) != 0;
-    Workspace w = carve((char *)workspace, N, S, K, !fused, m->weight_thres);
+    LM_REQUIRE(m->cap_valid >= 0 && m->cap_app >= 0, "negative workspace capacity");
+    Workspace w = carve((char *)workspace, N, S, K, !fused, m->weight_thres, m->cap_valid, m->cap_app);
     if (w.total > workspace_bytes)
         LM_FAIL(LM_ERR_WORKSPACE, "workspace has %zu bytes, %zu needed for N=%lld S=%d K=%d", workspace_bytes, w.total,
                 (long long)N, S, K);
@@ -250,7 +264,8 @@ int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *w
     mark(0);
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
     if (int rc = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
-                                      cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, st))
+                                      cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, (uint32_t)w.cap_valid,
+                                      cnt + LM_STAT_OVERFLOW, st))
         return rc;
     mark(LM_STAGE_CULL);
     if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS, (uint32_t)N, cnt + LM_STAT_QUEUE,
@@ -258,18 +273,21 @@ int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *w
         return rc;
     mark(LM_STAGE_DENSITY);
     if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.p_first, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
-                                     w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, row, st))
+                                     w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, row, (uint32_t)w.cap_app,
+                                     cnt + LM_STAT_OVERFLOW, st))
         return rc;
     mark(LM_STAGE_WEIGHTS);
     if (fused) {
-        if (int rc = lm_app_features(m, rays, w.app_idx, cnt, w.feat, st)) return rc;
+        if (int rc = lm_launch_app_features(m, rays, w.app_idx, cnt + LM_STAT_N_APP, (uint32_t)w.cap_app, w.feat, st)) return rc;
     } else {
         // channel counts the fused kernel does not cover: products through memory, then basis_mat
-        if (int rc = lm_app_products(m, rays, w.app_idx, cnt, w.products, st)) return rc;
-        if (int rc = lm_launch_basis(m->mlp_prec, m->mlp_packed, K, w.products, 0, cnt + LM_STAT_N_APP, w.feat, st)) return rc;
+        if (int rc = lm_launch_app_products(m, rays, w.app_idx, cnt + LM_STAT_N_APP, (uint32_t)w.cap_app, w.products, st)) return rc;
+        if (int rc = lm_launch_basis(m->mlp_prec, m->mlp_packed, K, w.products, 0, cnt + LM_STAT_N_APP, (uint32_t)w.cap_app, w.feat, st))
+            return rc;
     }
     mark(LM_STAGE_APP);
-    if (int rc = lm_launch_app_colour(m->mlp_prec, m->mlp_packed, K, S, w.feat, rays, w.app_idx, cnt + LM_STAT_N_APP, w.rgb, st))
+    if (int rc = lm_launch_app_colour(m->mlp_prec, m->mlp_packed, K, S, w.feat, rays, w.app_idx, cnt + LM_STAT_N_APP,
+                                      (uint32_t)w.cap_app, w.rgb, st))
         return rc;
     mark(LM_STAGE_COLOUR);
     if (int rc = lm_launch_composite(N, w.app_first, w.app_cnt, w.app_w, w.rgb, w.acc, m->white_bg, row, rgb_map, st)) return rc;

@@ -261,6 +261,16 @@ __device__ __forceinline__ void lm_ray_enqueue(bool mine, int bin, uint32_t r, u
     }
 }
 
+// A ray that asks for `cnt` entries from position `first` of a list with room for `cap`: true when it has
+// entries and they fit.  Rays that do not fit are counted in *overflow (one atomic per wave that has any) and
+// are treated by the caller as rays without entries.  Called by all lanes of the wave.
+__device__ __forceinline__ bool lm_ray_fits(uint32_t cnt, uint32_t first, uint32_t cap, uint32_t *overflow) {
+    const bool over = cnt != 0u && (uint64_t)first + cnt > (uint64_t)cap;
+    const uint64_t mask = __ballot(over);
+    if (mask != 0ull && (int)__lane_id() == __ffsll((unsigned long long)mask) - 1) atomicAdd(overflow, (uint32_t)__popcll(mask));
+    return cnt != 0u && !over;
+}
+
 // Visiting order of the whole-chunk render when the rays are image rows of length W (a
 // multiple of 8): position o -> ray index, 8 x 8 pixel tiles inside bands of 8 rows; the rays
 // behind the last full band keep their order.  A bijection on [0, N).

@@ -144,11 +144,11 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
 __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
                                                       const uint32_t *__restrict__ p_first,
                                                       const float *__restrict__ w_valid, float weight_thres,
-                                                      const uint32_t *__restrict__ app_cnt,
+                                                      uint32_t *__restrict__ app_cnt,
                                                       const uint32_t *__restrict__ p_end,
                                                       uint32_t *__restrict__ app_first, uint32_t *__restrict__ app_idx,
                                                       float *__restrict__ app_w, uint32_t *__restrict__ app_count,
-                                                      uint32_t row) {
+                                                      uint32_t row, uint32_t cap_app, uint32_t *__restrict__ overflow) {
     const unsigned lane = lm_lane();
     const uint64_t o = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     const uint64_t r = o < N ? lm_ray_order((uint32_t)o, (uint32_t)N, row) : o;
@@ -165,10 +165,16 @@ __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const u
         if (lane == 0) base = atomicAdd(app_count, total);
         base = __shfl(base, 0);
     }
-    if (r >= N) return;
     uint32_t slot = base + incl - cnt;
+    const bool fits = lm_ray_fits(cnt, slot, cap_app, overflow);
+    if (r >= N) return;
     app_first[r] = slot;
-    if (cnt) {
+    if (cnt && !fits) {
+        // no room for this ray's samples: it keeps the background colour (and is counted); the slots below the
+        // capacity that its range covers still get a sample index of this chunk and weight zero
+        app_cnt[r] = 0;
+        for (uint32_t i = slot; i < cap_app && i < slot + cnt; ++i) { app_idx[i] = (uint32_t)(r * (uint64_t)S); app_w[i] = 0.0f; }
+    } else if (cnt) {
         BitWalk it;
         it.start_at(bitmap, r * (uint64_t)S, (r + 1) * (uint64_t)S, p_first[r]);
         const uint32_t end = p_end[r];
@@ -245,11 +251,12 @@ int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
 }
 
 int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
-                        float weight_thres, const uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
-                        uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, hipStream_t stream) {
+                        float weight_thres, uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
+                        uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, uint32_t cap_app,
+                        uint32_t *overflow, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, p_first, w_valid,
-                       weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count, row);
+                       weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count, row, cap_app, overflow);
     LM_CHECK_LAUNCH("k_app_slots");
     return LM_OK;
 }

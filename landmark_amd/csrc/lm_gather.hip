@@ -484,9 +484,10 @@ __global__ __launch_bounds__(kBlock) void k_density_list(lm_geom g, PlaneSet ps,
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_app_list(lm_geom g, PlaneSet ps, int K, const float *__restrict__ rays,
                                                      const uint32_t *__restrict__ list,
-                                                     const uint32_t *__restrict__ count, float *__restrict__ out) {
+                                                     const uint32_t *__restrict__ count, uint32_t cap,
+                                                     float *__restrict__ out) {
     const unsigned qlane = threadIdx.x & 3u, slot = threadIdx.x >> 2;
-    const uint64_t M = *count;
+    const uint64_t M = min(*count, cap);  // the counter keeps counting past the list's capacity
     const uint64_t n_tiles = (M + kTile - 1) / kTile;
     for (uint64_t tile = lm_xcd_swizzle(blockIdx.x, gridDim.x); tile < n_tiles; tile += gridDim.x) {
         const uint64_t p = tile * kTile + slot;
@@ -661,7 +662,7 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
                                                                    const char *__restrict__ packed, lm_mma::PackLayout L,
                                                                    const float *__restrict__ rays,
                                                                    const uint32_t *__restrict__ list,
-                                                                   const uint32_t *__restrict__ count,
+                                                                   const uint32_t *__restrict__ count, uint32_t cap,
                                                                    float *__restrict__ feat) {
     using namespace lm_mma;
     using Mm = Mma<PREC>;
@@ -683,7 +684,7 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
     const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
     const unsigned qlane = lane & 3u, gs = lane >> 2;  // gather role: 4 lanes per sample, 16 samples per pass
     float *tile = reinterpret_cast<float *>(lds + basis_bytes + (threadIdx.x / LM_WAVE) * app_feat_tile_bytes(C));
-    const uint64_t M = *count;
+    const uint64_t M = min(*count, cap);  // the counter keeps counting past the list's capacity
     const uint64_t n_tiles = (M + 31) / 32;
     constexpr unsigned kWaves = AppFeatBlock<PREC>::N / LM_WAVE;
     const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * kWaves + threadIdx.x / LM_WAVE;
@@ -798,7 +799,7 @@ __global__ __launch_bounds__(AppFeatBlock<PREC>::N) void k_app_feat(lm_geom g, P
 
 template <int PREC, typename T>
 int launch_app_feat(int nu, const lm_model *m, const PlaneSet &ps, int K, const float *rays, const uint32_t *list,
-                    const uint32_t *count, float *feat, hipStream_t st) {
+                    const uint32_t *count, uint32_t cap, float *feat, hipStream_t st) {
     using namespace lm_mma;
     const PackLayout L = pack_layout(PREC, K);
     constexpr int kThreads = AppFeatBlock<PREC>::N;
@@ -819,7 +820,7 @@ int launch_app_feat(int nu, const lm_model *m, const PlaneSet &ps, int K, const 
             reserved = lds;                                                                                        \
         }                                                                                                          \
         hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, st, m->geom, ps, K, (const char *)m->mlp_packed, L, rays, \
-                           list, count, feat);                                                                     \
+                           list, count, cap, feat);                                                                \
         break;                                                                                                     \
     }
     switch (nu) {
@@ -962,23 +963,28 @@ extern "C" int lm_dense_alpha(const lm_model *m, const float *lin_x, const float
     return LM_OK;
 }
 
-extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
-                               float *products, void *stream) {
+// `count` entries of the list (at most `cap`, the list's capacity) -> products [count, K]
+int lm_launch_app_products(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *count, uint32_t cap,
+                           float *products, hipStream_t st) {
     LM_REQUIRE(m != nullptr, "model is null");
     if (int rc = lm_check_geom(&m->geom)) return rc;
     int dtype, K;
     if (int rc = lm_check_planes(m->app, m->n_planes, &dtype, &K)) return rc;
-    LM_REQUIRE(rays && app_idx && counters && products && lm_aligned16(products), "null or misaligned buffer");
+    LM_REQUIRE(rays && app_idx && count && products && lm_aligned16(products), "null or misaligned buffer");
     const PlaneSet ps = make_set(m->app, m->n_planes, &m->geom);
     const unsigned grid = (unsigned)lm_persistent_blocks(8);
     if (dtype == LM_F32)
-        hipLaunchKernelGGL(k_app_list<float>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, K, rays,
-                           app_idx, counters + LM_STAT_N_APP, products);
+        hipLaunchKernelGGL(k_app_list<float>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, K, rays, app_idx, count, cap, products);
     else
-        hipLaunchKernelGGL(k_app_list<__half>, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, m->geom, ps, K, rays,
-                           app_idx, counters + LM_STAT_N_APP, products);
+        hipLaunchKernelGGL(k_app_list<__half>, dim3(grid), dim3(kBlock), 0, st, m->geom, ps, K, rays, app_idx, count, cap, products);
     LM_CHECK_LAUNCH("k_app_list");
     return LM_OK;
+}
+
+extern "C" int lm_app_products(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
+                               float *products, void *stream) {
+    LM_REQUIRE(counters != nullptr, "counters is null");
+    return lm_launch_app_products(m, rays, app_idx, counters + LM_STAT_N_APP, UINT32_MAX, products, (hipStream_t)stream);
 }
 
 // True when the fused gather + basis_mat kernel covers this model's appearance planes.
@@ -991,28 +997,34 @@ int lm_app_feat_supported(const lm_model *m) {
 
 int lm_check_prec(int prec);
 int lm_check_K(int K);
+int lm_launch_app_features(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *cnt, uint32_t cap,
+                           float *feat, hipStream_t st);
 
 // appearance samples (list order) -> feat [n_app, 27] = basis_mat(plane * line products)
 extern "C" int lm_app_features(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *counters,
                                float *feat, void *stream) {
+    LM_REQUIRE(counters != nullptr, "counters is null");
+    return lm_launch_app_features(m, rays, app_idx, counters + LM_STAT_N_APP, UINT32_MAX, feat, (hipStream_t)stream);
+}
+
+int lm_launch_app_features(const lm_model *m, const float *rays, const uint32_t *app_idx, const uint32_t *cnt, uint32_t cap,
+                           float *feat, hipStream_t st) {
     LM_REQUIRE(m != nullptr, "model is null");
     if (int rc = lm_check_geom(&m->geom)) return rc;
     int dtype, K;
     if (int rc = lm_check_planes(m->app, m->n_planes, &dtype, &K)) return rc;
     if (int rc = lm_check_prec(m->mlp_prec)) return rc;
     if (int rc = lm_check_K(K)) return rc;
-    LM_REQUIRE(rays && app_idx && counters && feat, "null buffer");
+    LM_REQUIRE(rays && app_idx && cnt && feat, "null buffer");
     LM_REQUIRE(m->mlp_packed && lm_aligned16(m->mlp_packed), "packed colour-network weights are null or misaligned");
     if (!lm_app_feat_supported(m))
         LM_FAIL(LM_ERR_UNSUPPORTED, "fused appearance gather needs equal channel counts of 16..64 in steps of 16");
     const PlaneSet ps = make_set(m->app, m->n_planes, &m->geom);
     const int nu = m->app[0].C / 16;
-    hipStream_t st = (hipStream_t)stream;
-    const uint32_t *cnt = counters + LM_STAT_N_APP;
-#define LM_AF_GO(PREC_)                                                                                    \
-    return dtype == LM_F32 ? launch_app_feat<PREC_, float>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
-           : (nu & 1)      ? launch_app_feat<PREC_, Half4>(nu, m, ps, K, rays, app_idx, cnt, feat, st)     \
-                           : launch_app_feat<PREC_, __half>(nu, m, ps, K, rays, app_idx, cnt, feat, st)
+#define LM_AF_GO(PREC_)                                                                                         \
+    return dtype == LM_F32 ? launch_app_feat<PREC_, float>(nu, m, ps, K, rays, app_idx, cnt, cap, feat, st)     \
+           : (nu & 1)      ? launch_app_feat<PREC_, Half4>(nu, m, ps, K, rays, app_idx, cnt, cap, feat, st)     \
+                           : launch_app_feat<PREC_, __half>(nu, m, ps, K, rays, app_idx, cnt, cap, feat, st)
     switch (m->mlp_prec) {
         case LM_MLP_F32: LM_AF_GO(LM_MLP_F32);
         case LM_MLP_F16: LM_AF_GO(LM_MLP_F16);

@@ -389,7 +389,7 @@ __device__ __forceinline__ void stage_weights(char *lds, const char *packed, con
 template <int PREC, int MODE>
 __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restrict__ packed, PackLayout L,
                                                    const float *__restrict__ feat, const float *__restrict__ view,
-                                                   uint64_t M_host, const uint32_t *__restrict__ count, int S,
+                                                   uint64_t M_host, const uint32_t *__restrict__ count, uint32_t cap, int S,
                                                    const uint32_t *__restrict__ app_idx, float *__restrict__ rgb) {
     extern __shared__ __align__(16) char lds[];
     using Mm = Mma<PREC>;
@@ -402,7 +402,7 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
                                  : reinterpret_cast<const frag *>(packed + L.w3);
     const float *b1 = reinterpret_cast<const float *>(lds + P::kWeights), *b2 = b1 + 128, *b3 = b1 + 256;
     const unsigned lane = lm_lane(), j = lane & 31u, h = lane >> 5;
-    const uint64_t M = MODE == 0 ? M_host : (uint64_t)*count;
+    const uint64_t M = MODE == 0 ? M_host : (uint64_t)min(*count, cap);  // the counter keeps counting past the list's capacity
     constexpr int NCB = MlpBlock<PREC>::NCB, TILE = 32 * NCB;
     const uint64_t n_tiles = (M + TILE - 1) / TILE;
     const unsigned wpb = MlpBlock<PREC>::N / LM_WAVE;
@@ -462,8 +462,8 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
 template <int PREC>
 __global__ __launch_bounds__(256) void k_basis(const char *__restrict__ packed, PackLayout L, int K,
                                                const float *__restrict__ products, uint64_t M_host,
-                                               const uint32_t *__restrict__ count, float *__restrict__ feat) {
-    const uint64_t M = count ? (uint64_t)*count : M_host;
+                                               const uint32_t *__restrict__ count, uint32_t cap, float *__restrict__ feat) {
+    const uint64_t M = count ? (uint64_t)min(*count, cap) : M_host;
     using Mm = Mma<PREC>;
     using frag = typename Mm::frag;
     constexpr int G = Mm::G, CW = Mm::CW, NP = Mm::NP;
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(256) void k_basis(const char *__restrict__ packed, 
 
 template <int PREC, int MODE>
 int launch_mlp(const void *packed, int K, const float *feat, const float *view, uint64_t M, const uint32_t *count,
-               int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t stream) {
+               uint32_t cap, int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t stream) {
     const PackLayout L = pack_layout(PREC, K);
     const size_t lds = LdsPlan<PREC>::kBytes;
     static thread_local bool configured = false;
@@ -525,19 +525,19 @@ int launch_mlp(const void *packed, int K, const float *feat, const float *view, 
         configured = true;
     }
     hipLaunchKernelGGL((k_mlp<PREC, MODE>), dim3(grid), dim3(MlpBlock<PREC>::N), lds, stream, (const char *)packed, L, feat, view,
-                       M, count, S, app_idx, rgb);
+                       M, count, cap, S, app_idx, rgb);
     LM_CHECK_LAUNCH("k_mlp");
     return LM_OK;
 }
 
 template <int MODE>
 int dispatch_mlp(int prec, const void *packed, int K, const float *feat, const float *view, uint64_t M,
-                 const uint32_t *count, int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t st) {
+                 const uint32_t *count, uint32_t cap, int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t st) {
     switch (prec) {
-        case LM_MLP_F32: return launch_mlp<LM_MLP_F32, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
-        case LM_MLP_F16: return launch_mlp<LM_MLP_F16, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
-        case LM_MLP_BF16: return launch_mlp<LM_MLP_BF16, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
-        default: return launch_mlp<LM_MLP_F16X2, MODE>(packed, K, feat, view, M, count, S, app_idx, rgb, grid, st);
+        case LM_MLP_F32: return launch_mlp<LM_MLP_F32, MODE>(packed, K, feat, view, M, count, cap, S, app_idx, rgb, grid, st);
+        case LM_MLP_F16: return launch_mlp<LM_MLP_F16, MODE>(packed, K, feat, view, M, count, cap, S, app_idx, rgb, grid, st);
+        case LM_MLP_BF16: return launch_mlp<LM_MLP_BF16, MODE>(packed, K, feat, view, M, count, cap, S, app_idx, rgb, grid, st);
+        default: return launch_mlp<LM_MLP_F16X2, MODE>(packed, K, feat, view, M, count, cap, S, app_idx, rgb, grid, st);
     }
 }
 
@@ -598,13 +598,13 @@ extern "C" int lm_mlp(int32_t prec, const void *packed, int32_t K, const float *
     LM_REQUIRE(M >= 0, "negative count");
     if (M == 0) return LM_OK;
     LM_REQUIRE(packed && feat && view && rgb && lm_aligned16(packed), "null or misaligned buffer");
-    return dispatch_mlp<0>(prec, packed, K, feat, view, (uint64_t)M, nullptr, 1, nullptr, rgb, mlp_grid((uint64_t)M),
+    return dispatch_mlp<0>(prec, packed, K, feat, view, (uint64_t)M, nullptr, 0u, 1, nullptr, rgb, mlp_grid((uint64_t)M),
                            (hipStream_t)stream);
 }
 
 // products [M,K] -> feat [M,27]; M from the host, or from *count when count != NULL
 int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
-                    float *feat, hipStream_t st) {
+                    uint32_t cap, float *feat, hipStream_t st) {
     if (int rc = lm_check_prec(prec)) return rc;
     if (int rc = lm_check_K(K)) return rc;
     LM_REQUIRE(packed && products && feat && lm_aligned16(packed) && lm_aligned16(products), "null or misaligned buffer");
@@ -613,10 +613,10 @@ int lm_launch_basis(int prec, const void *packed, int K, const float *products, 
     const unsigned grid = count ? (unsigned)lm_persistent_blocks(4)
                                 : (unsigned)std::min<uint64_t>(std::max<uint64_t>((tiles + 3) / 4, 1), (uint64_t)lm_persistent_blocks(4));
     switch (prec) {
-        case LM_MLP_F32: hipLaunchKernelGGL(k_basis<LM_MLP_F32>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
-        case LM_MLP_F16: hipLaunchKernelGGL(k_basis<LM_MLP_F16>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
-        case LM_MLP_BF16: hipLaunchKernelGGL(k_basis<LM_MLP_BF16>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
-        default: hipLaunchKernelGGL(k_basis<LM_MLP_F16X2>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, feat); break;
+        case LM_MLP_F32: hipLaunchKernelGGL(k_basis<LM_MLP_F32>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, cap, feat); break;
+        case LM_MLP_F16: hipLaunchKernelGGL(k_basis<LM_MLP_F16>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, cap, feat); break;
+        case LM_MLP_BF16: hipLaunchKernelGGL(k_basis<LM_MLP_BF16>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, cap, feat); break;
+        default: hipLaunchKernelGGL(k_basis<LM_MLP_F16X2>, dim3(grid), dim3(256), 0, st, (const char *)packed, L, K, products, M, count, cap, feat); break;
     }
     LM_CHECK_LAUNCH("k_basis");
     return LM_OK;
@@ -626,14 +626,14 @@ extern "C" int lm_basis(int32_t prec, const void *packed, int32_t K, const float
                         void *stream) {
     LM_REQUIRE(M >= 0, "negative count");
     if (M == 0) return LM_OK;
-    return lm_launch_basis(prec, packed, K, products, (uint64_t)M, nullptr, feat, (hipStream_t)stream);
+    return lm_launch_basis(prec, packed, K, products, (uint64_t)M, nullptr, 0u, feat, (hipStream_t)stream);
 }
 
 // used by lm_render: feat [n_app,27] + ray directions -> rgb [n_app,3]
 int lm_launch_app_colour(int prec, const void *packed, int K, int S, const float *feat, const float *rays,
-                         const uint32_t *app_idx, const uint32_t *count, float *rgb, hipStream_t stream) {
+                         const uint32_t *app_idx, const uint32_t *count, uint32_t cap, float *rgb, hipStream_t stream) {
     if (int rc = lm_check_prec(prec)) return rc;
     if (int rc = lm_check_K(K)) return rc;
     LM_REQUIRE(packed && lm_aligned16(packed), "packed colour-network weights are null or misaligned");
-    return dispatch_mlp<1>(prec, packed, K, feat, rays, 0, count, S, app_idx, rgb, (unsigned)lm_persistent_blocks(1), stream);
+    return dispatch_mlp<1>(prec, packed, K, feat, rays, 0, count, cap, S, app_idx, rgb, (unsigned)lm_persistent_blocks(1), stream);
 }

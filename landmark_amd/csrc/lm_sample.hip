@@ -165,7 +165,8 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
                                                             uint32_t *__restrict__ ray_list, uint32_t *__restrict__ bins,
                                                             uint32_t *__restrict__ n_valid, float *__restrict__ acc,
                                                             float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
-                                                            uint32_t *__restrict__ p_end) {
+                                                            uint32_t *__restrict__ p_end, uint32_t cap_valid,
+                                                            uint32_t *__restrict__ overflow) {
     __shared__ uint32_t s_cnt[kBlock];
     const unsigned lane = lm_lane(), wave = threadIdx.x / LM_WAVE;
     constexpr unsigned kRays = kBlock / WPR;
@@ -196,9 +197,9 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
         if (lane == 0) base = atomicAdd(n_valid, total);
         base = __shfl(base, 0);
     }
-    const bool any = cnt != 0;
+    const uint32_t first = base + incl - cnt;
+    const bool any = lm_ray_fits(cnt, first, cap_valid, overflow);
     if (r < N) {
-        const uint32_t first = base + incl - cnt;
         p_first[r] = first;
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
     }
@@ -219,7 +220,8 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
                                                                    uint32_t *__restrict__ bins,
                                                                    uint32_t *__restrict__ n_valid, float *__restrict__ acc,
                                                                    float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
-                                                                   uint32_t *__restrict__ p_end) {
+                                                                   uint32_t *__restrict__ p_end, uint32_t cap_valid,
+                                                                   uint32_t *__restrict__ overflow) {
     const unsigned lane = lm_lane();
     const unsigned sub = threadIdx.x % LPR;  // this lane's share of its ray's words
     const uint64_t o = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / LPR;  // position in the visiting order
@@ -255,9 +257,10 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
         if (lane == 0) base = atomicAdd(n_valid, total);
         base = __shfl(base, 0);
     }
-    const bool any = cnt != 0, mine = r < N && sub == 0;
+    const bool mine = r < N && sub == 0;
+    const uint32_t first = base + incl - cnt;
+    const bool any = lm_ray_fits(mine ? cnt : 0u, first, cap_valid, overflow);
     if (mine) {
-        const uint32_t first = base + incl - cnt;
         p_first[r] = first;
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
     }
@@ -509,12 +512,14 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
 // count is not a multiple of 64).
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *bins, uint32_t *n_valid, float *acc, float *depth,
-                         uint32_t *app_cnt, uint32_t *p_end, uint32_t row, hipStream_t st) {
+                         uint32_t *app_cnt, uint32_t *p_end, uint32_t row, uint32_t cap_valid, uint32_t *overflow,
+                         hipStream_t st) {
     const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
     LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
 #define LM_CULL_SETUP(W_)                                                                                             \
     hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3((unsigned)(((uint64_t)N * W_ + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, \
-                       *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt, p_end)
+                       *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt, p_end,  \
+                       cap_valid, overflow)
     if (wpr == 1) {
         LM_CULL_SETUP(1);
     } else if (wpr == 2) {
@@ -532,7 +537,7 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
 #define LM_CULL_SERIAL(L_)                                                                                           \
     hipLaunchKernelGGL(k_cull_rays_setup_serial<L_>, dim3((unsigned)(((uint64_t)N * L_ + kBlock - 1) / kBlock)),         \
                        dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, \
-                       depth, app_cnt, p_end)
+                       depth, app_cnt, p_end, cap_valid, overflow)
         switch (lpr) {
             case 1: LM_CULL_SERIAL(1); break;
             case 2: LM_CULL_SERIAL(2); break;

@@ -46,6 +46,7 @@ class GridNeRFHIP:
         term_eps: float = 0.0,
         release_source: bool = False,
         occupancy: str = "auto",  # auto | cells | u8 | f32: storage of the occupancy volume
+        capacity: str = "adaptive",  # adaptive | worst: how the render workspace is sized (see `capacities`)
     ):
         if not torch.cuda.is_available():
             raise L.LandmarkError("GridNeRFHIP needs a GPU; there is no CPU path")
@@ -54,6 +55,11 @@ class GridNeRFHIP:
         self.p = params
         self.mlp_precision = mlp_precision
         self.term_eps = float(term_eps)
+        if capacity not in ("adaptive", "worst"):
+            raise ValueError(f"capacity {capacity!r}")
+        self.capacity = capacity
+        # [valid, appearance] samples per ray the workspace is sized for (chunk average); grows on overflow
+        self.samples_per_ray = [32.0, 12.0]
         # set by callers that render images: rays arrive row by row, this many per row (0 = unknown); lets the
         # kernels visit rays in 8 x 8 pixel tiles.  Results do not depend on it.
         self.ray_row_length = 0
@@ -287,15 +293,17 @@ class GridNeRFHIP:
         self._geom_cache[S] = (g, (a_d, t_d))
         return g
 
-    def _model_struct(self, S: int, white_bg: bool) -> L.LmModel:
-        """The lm_model of a render with S samples per ray, built once per distinct setting and reused (a caller
-        that keeps small chunks pays for launches only); never carries event handles."""
-        key = (int(S), bool(white_bg), self.mlp_precision, float(self.term_eps), int(self.ray_row_length), id(self._geom_cache))
+    def _model_struct(self, S: int, white_bg: bool, caps: Tuple[int, int] = (0, 0)) -> L.LmModel:
+        """The lm_model of a render with S samples per ray and workspace capacities `caps` (valid samples,
+        appearance samples; 0 = worst case), built once per distinct setting and reused (a caller that keeps
+        small chunks pays for launches only); never carries event handles."""
+        key = (int(S), bool(white_bg), self.mlp_precision, float(self.term_eps), int(self.ray_row_length), caps)
         m = self._struct_cache.get(key)
         if m is None:
             if len(self._struct_cache) > 64:
                 self._struct_cache.clear()
             m = self._struct_cache[key] = self._build_model_struct(S, white_bg)
+            m.cap_valid, m.cap_app = int(caps[0]), int(caps[1])
         return m
 
     def _build_model_struct(self, S: int, white_bg: bool) -> L.LmModel:
@@ -322,14 +330,41 @@ class GridNeRFHIP:
             return int(self.p.n_importance)
         return int(N_samples) if N_samples > 0 else int(self.nSamples)
 
-    def workspace(self, n_rays: int, S: int, slot: int = 0) -> torch.Tensor:
+    # ------------------------------------------------------------------ workspace
+    def capacities(self, n_rays: int, S: int) -> Tuple[int, int]:
+        """Room (valid samples, appearance samples) the workspace of an n_rays chunk is given.  With
+        `capacity="worst"` both are 0 = the worst case, which cannot overflow (every sample valid, every ray with
+        min(S, 1 / weight threshold) appearance samples: 132 bytes per ray and sample).  Otherwise they follow
+        `samples_per_ray` = [valid, appearance] samples per ray averaged over a chunk, which starts from a guess
+        and is raised whenever a render reports an overflow (`forward` and `render_frame` repeat such a chunk)."""
+        if self.capacity == "worst":
+            return (0, 0)
+        total = int(n_rays) * int(S)
+        per_ray_app = min(int(S), int(1.001 / self.p.rayMarch_weight_thres) + 2) if self.p.rayMarch_weight_thres > 0 else int(S)
+        want_valid = max(1 << 16, int(self.samples_per_ray[0] * n_rays) + 1)
+        want_app = max(1 << 14, int(self.samples_per_ray[1] * n_rays) + 1)
+        cap_valid = 0 if want_valid >= total else want_valid
+        cap_app = 0 if want_app >= int(n_rays) * per_ray_app else want_app
+        return (cap_valid, cap_app)
+
+    def _grow_capacity(self, n_rays: int, n_valid: int, n_app: int, valid_overflowed: bool) -> None:
+        """Raise samples_per_ray so that a chunk like the one that reported these counts fits, with a quarter to spare.
+        After a valid-sample overflow the appearance count is only a lower bound: double it as well."""
+        v = 1.25 * n_valid / max(n_rays, 1)
+        a = 1.25 * n_app / max(n_rays, 1)
+        if valid_overflowed:
+            a = max(a, 2.0 * self.samples_per_ray[1])
+        self.samples_per_ray = [max(self.samples_per_ray[0], v), max(self.samples_per_ray[1], a)]
+
+    def workspace(self, n_rays: int, S: int, slot: int = 0, caps: Optional[Tuple[int, int]] = None) -> torch.Tensor:
         """Device workspace for chunks of up to n_rays rays; grown on demand and reused
         (the role of allocate_tensors, dist_render/kernel/cuda_render_extend.py:35-159).
         Renders that run concurrently on different streams take different slots."""
-        key = (int(n_rays), int(S), self.mlp_precision)
+        caps = self.capacities(n_rays, S) if caps is None else caps
+        key = (int(n_rays), int(S), self.mlp_precision, caps)
         need = self._need_cache.get(key)
         if need is None:
-            m = self._model_struct(S, True)
+            m = self._model_struct(S, True, caps)
             need = self.lib.lm_render_workspace_bytes(C.byref(m), n_rays)
             if need == 0:
                 raise L.LandmarkError(self.lib.lm_last_error().decode())
@@ -350,8 +385,8 @@ class GridNeRFHIP:
         (large launches are what keeps the GPU busy: a 1080p frame in 4096-ray chunks takes 14
         times as long as in two chunks), as many as `workspace_budget` and 32-bit sample indices allow."""
         S = self._samples_for(N_samples)
-        m = self._model_struct(S, True)
         probe = 1 << 16
+        m = self._model_struct(S, True, self.capacities(probe, S))
         per_ray = self.lib.lm_render_workspace_bytes(C.byref(m), probe) / probe
         fit = int(self.workspace_budget / max(per_ray, 1.0))
         cap = min(1 << 20, ((1 << 32) - 1) // S, max(fit, 4096))
@@ -393,25 +428,62 @@ class GridNeRFHIP:
         rgb = torch.empty((N, 3), dtype=torch.float32, device=self.device)
         depth = torch.empty((N,), dtype=torch.float32, device=self.device)
         step = self.preferred_chunk(N, N_samples) if N else 1  # a call of any size: split where one launch cannot take it
-        for start in range(0, N, step):
+        starts = list(range(0, N, step))
+        counters = torch.zeros((max(len(starts), 1), L.LM_STAT_WORDS), dtype=torch.int32, device=self.device)
+        for ci, start in enumerate(starts):
             sl = slice(start, min(start + step, N))
-            self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples)
+            self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, counters=counters[ci])
+        self.finish_chunks([(slice(st, min(st + step, N)), counters[ci]) for ci, st in enumerate(starts)], rays, rgb, depth,
+                           white_bg=white_bg, N_samples=N_samples)
+        if starts:
+            self.counters.copy_(counters[len(starts) - 1])
         return {"rgb_map": rgb, "depth_map": depth}, {}
 
     __call__ = forward
+
+    def finish_chunks(self, chunks, rays, rgb, depth, white_bg=True, N_samples=-1) -> int:
+        """Chunks rendered with a workspace below the worst case may have dropped rays: read their counter blocks
+        (one small copy, the call's one host synchronisation), raise the capacity to what the counters ask for and
+        render the affected chunks again until none overflows.  `chunks`: (slice of the ray array, the counter
+        block its render wrote).  Returns the number of repeated renders; nothing to do with capacity="worst"."""
+        if self.capacity == "worst" or not chunks:
+            return 0
+        repeats = 0
+        pending = list(chunks)
+        for _ in range(6):
+            host = torch.stack([c for _, c in pending]).cpu().long() & 0xFFFFFFFF
+            again = []
+            for (sl, cnt), row in zip(pending, host):
+                if int(row[L.LM_STAT_OVERFLOW]) == 0:
+                    continue
+                n = sl.stop - sl.start
+                S = self._samples_for(N_samples)
+                caps = self.capacities(n, S)
+                valid_over = caps[0] != 0 and int(row[L.LM_STAT_N_VALID]) > caps[0]
+                self._grow_capacity(n, int(row[L.LM_STAT_N_VALID]), int(row[L.LM_STAT_N_APP]), valid_over)
+                again.append((sl, cnt))
+            if not again:
+                return repeats
+            for sl, cnt in again:
+                self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, counters=cnt)
+                repeats += 1
+            pending = again
+        raise L.LandmarkError("workspace capacity still overflows after six repeats")
 
     def render_into(self, rays, rgb, depth, white_bg=True, N_samples=-1, counters=None, events=None, slot=0):
         """lm_render on device tensors the caller owns.  `counters`: int32[LM_STAT_WORDS] device tensor
         receiving the chunk's sample counts; `events`: 7 recorded torch.cuda.Event objects
         (enable_timing=True) re-recorded around the stages on the current stream.  Calls that may
         run at the same time (different streams) must use different slots: a slot owns a workspace
-        and a counter block."""
+        and a counter block.  The workspace has the room `capacities` gives it: unless that is the worst
+        case, counters[LM_STAT_OVERFLOW] tells whether rays were dropped (see finish_chunks)."""
         N = rays.shape[0]
         if N == 0:
             return
         S = self._samples_for(N_samples)
-        ws = self.workspace(N, S, slot)
-        m = self._model_struct(S, white_bg)
+        caps = self.capacities(N, S)
+        ws = self.workspace(N, S, slot, caps)
+        m = self._model_struct(S, white_bg, caps)
         if events is not None:
             m = L.LmModel.from_buffer_copy(m)  # the cached struct stays free of event handles
             for i, e in enumerate(events):
@@ -477,7 +549,8 @@ class GridNeRFHIP:
     def last_counts(self) -> Dict[str, int]:
         """Valid / appearance sample counts of the last chunk (synchronises)."""
         c = self.counters.cpu()
-        return {"n_valid": int(c[L.LM_STAT_N_VALID]) & 0xFFFFFFFF, "n_app": int(c[L.LM_STAT_N_APP]) & 0xFFFFFFFF}
+        return {"n_valid": int(c[L.LM_STAT_N_VALID]) & 0xFFFFFFFF, "n_app": int(c[L.LM_STAT_N_APP]) & 0xFFFFFFFF,
+                "overflow": int(c[L.LM_STAT_OVERFLOW]) & 0xFFFFFFFF}
 
     # ------------------------------------------------------------------ stage entry points
     @torch.no_grad()

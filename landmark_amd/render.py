@@ -143,6 +143,7 @@ def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 20, app_cod
     current = torch.cuda.current_stream(gridnerf.device)
     side = gridnerf.side_streams(min(int(streams), len(starts)) - 1) if streams > 1 and len(starts) > 1 else []
     gridnerf._set_app_code(gridnerf.mlp_precision, app_code)
+    counters = torch.zeros((len(starts), 16), dtype=torch.int32, device=gridnerf.device)  # one block per chunk
     if side:
         ready = torch.cuda.Event()
         ready.record(current)
@@ -152,13 +153,16 @@ def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 20, app_cod
     saved = gridnerf.ray_row_length
     gridnerf.ray_row_length = W if W % 8 == 0 else 0
     try:
+        done = []
         for i, start in enumerate(starts):
             sl = slice(start, min(start + chunk, N))
             with torch.cuda.stream(lanes[i % len(lanes)]):
-                gridnerf.render_into(rays[sl], rgb[sl], dep[sl], white_bg=white_bg, slot=i % len(lanes))
-    finally:
-        gridnerf.ray_row_length = saved
+                gridnerf.render_into(rays[sl], rgb[sl], dep[sl], white_bg=white_bg, slot=i % len(lanes), counters=counters[i])
+            done.append((sl, counters[i]))
         for s in side:
             current.wait_stream(s)
+        gridnerf.finish_chunks(done, rays, rgb, dep, white_bg=white_bg)  # repeats chunks whose workspace overflowed
+    finally:
+        gridnerf.ray_row_length = saved
     image = postprocess_rgba8(rgb, H, W, host_image)
     return (image, dep.view(H, W)) if depth else image

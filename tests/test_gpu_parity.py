@@ -487,7 +487,7 @@ def test_chunk_drivers(gpu_lib):
     # the library's own choice of chunk: everything at once here, bounded by the workspace budget and by
     # 32-bit sample indices; a single call larger than that is split inside forward
     assert m.preferred_chunk(rays.shape[0]) == rays.shape[0] and m.preferred_chunk(1 << 30) == 1 << 20
-    small = _model(p)
+    small = _model(p, capacity="worst")
     small.workspace_budget = 5000 * small.lib.lm_render_workspace_bytes(C.byref(small._model_struct(64, True)), 1 << 16) // (1 << 16)
     more = scenes.pinhole_rays(80, 80, 80.0, scenes.sphere_pose(2.5, 5))
     assert 4096 <= small.preferred_chunk(more.shape[0]) < more.shape[0]
@@ -500,6 +500,59 @@ def test_chunk_drivers(gpu_lib):
     assert torch.equal(ret["rgb_map"], full["rgb_map"][:512])
     with pytest.raises(NotImplementedError):
         m(rays, is_train=True)
+
+
+@pytest.mark.parametrize("opt,S", [(1, 128), (0, 200)])
+def test_workspace_capacity_overflow_is_reported_and_repeatable(gpu_lib, opt, S):
+    """A workspace below the worst case: rays whose samples do not fit are dropped and counted, the counters still
+    report what would have fit, and the repeat with those capacities equals the worst-case render bit for bit."""
+    from landmark_amd import _lib as L
+
+    p = _scene(opt=opt, S=S, thre=0.0, step_ratio=0.3)
+    rays = scenes.pinhole_rays(100, 90, 85.0, scenes.sphere_pose(2.5, 9)).cuda()
+    N = rays.shape[0]
+    m = _model(p, capacity="worst")
+    full, _ = m(rays, N_samples=S)
+    want = m.last_counts()
+    assert want["overflow"] == 0 and want["n_app"] > 1000
+
+    def render(caps):
+        st = L.LmModel.from_buffer_copy(m._model_struct(S, True))
+        st.cap_valid, st.cap_app = caps
+        need = m.lib.lm_render_workspace_bytes(C.byref(st), N)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        rgb, dep = torch.empty((N, 3), device="cuda"), torch.empty((N,), device="cuda")
+        cnt = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device="cuda")
+        L.check(m.lib.lm_render(C.byref(st), rays.data_ptr(), N, ws.data_ptr(), need, rgb.data_ptr(), dep.data_ptr(), cnt.data_ptr(),
+                                L.current_stream()), "lm_render")
+        torch.cuda.synchronize()
+        c = cnt.cpu().long() & 0xFFFFFFFF
+        return rgb, dep, int(c[L.LM_STAT_N_VALID]), int(c[L.LM_STAT_N_APP]), int(c[L.LM_STAT_OVERFLOW]), need
+
+    worst_bytes = m.lib.lm_render_workspace_bytes(C.byref(m._model_struct(S, True)), N)
+    # room for a third of the valid samples: rays are dropped, the valid count is still the whole chunk's
+    rgb, dep, nv, na, over, need = render((want["n_valid"] // 3, want["n_app"]))
+    assert over > 0 and nv == want["n_valid"] and na < want["n_app"] and need < worst_bytes
+    kept = (rgb == full["rgb_map"]).all(-1) & (dep == full["depth_map"])
+    dropped = ~kept
+    assert int(dropped.sum()) <= over and bool((rgb[dropped] == 1.0).all()) and bool((dep[dropped] == 0.0).all())
+    # room for half of the appearance samples: those rays keep their depth and show the background
+    rgb, dep, nv, na, over, _ = render((want["n_valid"], want["n_app"] // 2))
+    assert over > 0 and nv == want["n_valid"] and na == want["n_app"]
+    assert torch.equal(dep, full["depth_map"]) and not torch.equal(rgb, full["rgb_map"])
+    # exactly enough room: nothing dropped, identical bits
+    rgb, dep, nv, na, over, _ = render((want["n_valid"], want["n_app"]))
+    assert over == 0 and torch.equal(rgb, full["rgb_map"]) and torch.equal(dep, full["depth_map"])
+    # the wrapper's adaptive sizing: starts too small, reads the counters, repeats the chunk, remembers
+    a = _model(p)
+    a.samples_per_ray = [0.2 * want["n_valid"] / N, 0.2 * want["n_app"] / N]
+    assert a.capacities(N, S)[0] * 4 < want["n_valid"] * 4 and a.capacities(N, S) != (0, 0)
+    out, _ = a(rays, N_samples=S)
+    assert torch.equal(out["rgb_map"], full["rgb_map"]) and torch.equal(out["depth_map"], full["depth_map"])
+    assert a.samples_per_ray[0] * N >= want["n_valid"] and a.samples_per_ray[1] * N >= want["n_app"]
+    assert a.last_counts()["overflow"] == 0
+    out2, _ = a(rays, N_samples=S)  # now sized right the first time
+    assert torch.equal(out2["rgb_map"], full["rgb_map"])
 
 
 @pytest.mark.parametrize("S,width", [(128, 96), (64, 40), (100, 96), (128, 50)])

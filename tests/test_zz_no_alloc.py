@@ -55,7 +55,7 @@ def test_static_workspace_render_equals_lm_render(gpu_lib, opt, S):
     from landmark_amd.model import GridNeRFHIP
 
     p = _scene(S, opt)
-    model = GridNeRFHIP(p, mlp_precision="f16x2")
+    model = GridNeRFHIP(p, mlp_precision="f16x2", capacity="worst")
     big = scenes.pinhole_rays(60, 50, 52.0, scenes.sphere_pose(2.5, 9)).cuda()  # 3000 rays
     small = big[1234:1234 + 517].contiguous()
     for rays in (big, small, big):  # the second call is smaller than the first and finds its leftovers
@@ -76,7 +76,7 @@ def test_static_workspace_refuses_oversized_chunks(gpu_lib):
     from landmark_amd.model import GridNeRFHIP
 
     p = _scene(128, 1)
-    model = GridNeRFHIP(p)
+    model = GridNeRFHIP(p, capacity="worst")
     lib = model.lib
     m = model._model_struct(128, True)
     N = 1 << 16  # 65536 rays x 128 samples: far beyond the built-in array
