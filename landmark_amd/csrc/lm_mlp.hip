@@ -186,6 +186,18 @@ __device__ __forceinline__ void sincos_f32(float x, float &s, float &c) {
     c = ((q + 1) & 2) ? -cc : cc;
 }
 
+// sin and cos through the hardware functions (argument in revolutions) after a two-constant reduction by
+// 2 pi: within 4.3e-7 of the exact values for |x| <= 8192 (measured over 2^24 arguments per range), seven
+// instructions per value.  Used by the split-fp16 mode, whose products carry about 21 mantissa bits anyway.
+__device__ __forceinline__ void sincos_hw(float x, float &s, float &c) {
+    const float k = rintf(x * 0.15915494309189535f);
+    float r = fmaf(-k, 6.28125f, x);
+    r = fmaf(-k, 1.9353071795864769e-3f, r);
+    const float t = r * 0.15915494309189535f;
+    s = __builtin_amdgcn_sinf(t);
+    c = __builtin_amdgcn_cosf(t);
+}
+
 // One dense layer on the wave's 32*NCB samples: acc[fb][cb] (+)= W[32*fb .. +32, :] x B[cb]
 // for NB row blocks and NCB column blocks of 32 samples.  Every weight fragment read from
 // LDS feeds NCB MFMAs (an A fragment is 1 KB per 32-cycle MFMA, which is exactly the LDS
@@ -262,12 +274,59 @@ __device__ __forceinline__ void relu_to_frags(const floatx16 &acc, typename Mma<
     }
 }
 
-// raw[cb][16] (the lane's 16 input rows of each of its NCB samples) -> rgb in out[cb][0..2]
-// (meaningful on lanes with h == 0)
+// raw[cb][16] (the lane's 16 input rows of each of its NCB samples) -> the first layer's B fragments: per lane
+// five groups of 16 slots (raw, sin, cos, sin 2x, cos 2x)
 template <int PREC, int NCB>
-__device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w1, const typename Mma<PREC>::frag *w2,
-                                               const typename Mma<PREC>::frag *w3, const float *b1, const float *b2,
-                                               const float *b3, const float (*raw)[16], unsigned lane, float (*out)[3]) {
+__device__ __forceinline__ void encode_inputs(const float (*raw)[16],
+                                              typename Mma<PREC>::frag (*bfrag)[kSlots1 / Mma<PREC>::G][Mma<PREC>::NP]) {
+    using M = Mma<PREC>;
+    constexpr int G = M::G, T1 = kSlots1 / G;
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb) {
+        float slots[kSlots1];
+        constexpr bool kExact = PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2;
+        bool big = false;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float x = raw[cb][v];
+            float s1, c1;
+            if (PREC == LM_MLP_F16X2) {
+                sincos_hw(x, s1, c1);
+                big |= fabsf(x) > kSincosMax;
+            } else if (kExact) {
+                sincos_f32(x, s1, c1);
+                big |= fabsf(x) > kSincosMax;
+            } else {
+                s1 = __sinf(x); c1 = __cosf(x);
+            }
+            const float s2 = 2.0f * s1 * c1;
+            const float c2 = fmaf(-2.0f * s1, s1, 1.0f);
+            slots[v] = x; slots[16 + v] = s1; slots[32 + v] = c1; slots[48 + v] = s2; slots[64 + v] = c2;
+        }
+        if (kExact && __builtin_expect(big, 0)) {
+            // arguments beyond the fast reduction's range: library routines, rarely if ever taken
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float x = raw[cb][v];
+                if (fabsf(x) > kSincosMax) {
+                    const float s1 = sinf(x), c1 = cosf(x);
+                    slots[16 + v] = s1; slots[32 + v] = c1;
+                    slots[48 + v] = 2.0f * s1 * c1; slots[64 + v] = fmaf(-2.0f * s1, s1, 1.0f);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < T1; ++t) M::pack(slots + t * G, bfrag[cb][t]);
+    }
+}
+
+// first-layer B fragments -> rgb in out[cb][0..2] (meaningful on lanes with h == 0)
+template <int PREC, int NCB>
+__device__ __forceinline__ void colour_layers(const typename Mma<PREC>::frag *w1, const typename Mma<PREC>::frag *w2,
+                                              const typename Mma<PREC>::frag *w3, const float *b1, const float *b2,
+                                              const float *b3,
+                                              const typename Mma<PREC>::frag (*bfrag)[kSlots1 / Mma<PREC>::G][Mma<PREC>::NP],
+                                              unsigned lane, float (*out)[3]) {
     using M = Mma<PREC>;
     using frag = typename M::frag;
     constexpr int G = M::G, NP = M::NP;
@@ -277,55 +336,18 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
     constexpr int PF = G == 1 ? 4 : 1;
     const unsigned h = lane >> 5;
     frag b2frag[NCB][T2][NP];
-    {
-        frag bfrag[NCB][T1][NP];
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
-            float slots[kSlots1];
-            constexpr bool kExact = PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2;
-            bool big = false;
+    for (int pass = 0; pass < 4 / NB; ++pass) {
+        floatx16 acc[NB][NCB];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float x = raw[cb][v];
-                float s1, c1;
-                if (kExact) {
-                    sincos_f32(x, s1, c1);
-                    big |= fabsf(x) > kSincosMax;
-                } else {
-                    s1 = __sinf(x); c1 = __cosf(x);
-                }
-                const float s2 = 2.0f * s1 * c1;
-                const float c2 = fmaf(-2.0f * s1, s1, 1.0f);
-                slots[v] = x; slots[16 + v] = s1; slots[32 + v] = c1; slots[48 + v] = s2; slots[64 + v] = c2;
-            }
-            if (kExact && __builtin_expect(big, 0)) {
-                // arguments beyond the fast reduction's range: library routines, rarely if ever taken
+        for (int fb = 0; fb < NB; ++fb)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const float x = raw[cb][v];
-                    if (fabsf(x) > kSincosMax) {
-                        const float s1 = sinf(x), c1 = cosf(x);
-                        slots[16 + v] = s1; slots[32 + v] = c1;
-                        slots[48 + v] = 2.0f * s1 * c1; slots[64 + v] = fmaf(-2.0f * s1, s1, 1.0f);
-                    }
-                }
-            }
+            for (int cb = 0; cb < NCB; ++cb) acc[fb][cb] = load_bias(b1, (pass * NB + fb) * 2 + h);
+        dense_layer<PREC, NB, NCB, T1, PF>(w1, pass * NB, lane, bfrag, acc);
 #pragma unroll
-            for (int t = 0; t < T1; ++t) M::pack(slots + t * G, bfrag[cb][t]);
-        }
+        for (int fb = 0; fb < NB; ++fb)
 #pragma unroll
-        for (int pass = 0; pass < 4 / NB; ++pass) {
-            floatx16 acc[NB][NCB];
-#pragma unroll
-            for (int fb = 0; fb < NB; ++fb)
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) acc[fb][cb] = load_bias(b1, (pass * NB + fb) * 2 + h);
-            dense_layer<PREC, NB, NCB, T1, PF>(w1, pass * NB, lane, bfrag, acc);
-#pragma unroll
-            for (int fb = 0; fb < NB; ++fb)
-#pragma unroll
-                for (int cb = 0; cb < NCB; ++cb) relu_to_frags<PREC>(acc[fb][cb], &b2frag[cb][(pass * NB + fb) * (16 / G)]);
-        }
+            for (int cb = 0; cb < NCB; ++cb) relu_to_frags<PREC>(acc[fb][cb], &b2frag[cb][(pass * NB + fb) * (16 / G)]);
     }
     frag b3frag[NCB][T2][NP];
 #pragma unroll
@@ -348,7 +370,11 @@ __device__ __forceinline__ void colour_network(const typename Mma<PREC>::frag *w
 #pragma unroll
     for (int cb = 0; cb < NCB; ++cb)
 #pragma unroll
-        for (int k = 0; k < 3; ++k) out[cb][k] = 1.0f / (1.0f + expf(-acc3[0][cb][k]));
+        for (int k = 0; k < 3; ++k) {
+            // sigmoid; the hardware reciprocal is within one unit in the last place, enough for every mode
+            const float e = (PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2) ? expf(-acc3[0][cb][k]) : __expf(-acc3[0][cb][k]);
+            out[cb][k] = __builtin_amdgcn_rcpf(1.0f + e);
+        }
 }
 
 template <int PREC> struct LdsPlan {
@@ -390,7 +416,8 @@ template <int PREC, int MODE>
 __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restrict__ packed, PackLayout L,
                                                    const float *__restrict__ feat, const float *__restrict__ view,
                                                    uint64_t M_host, const uint32_t *__restrict__ count, uint32_t cap, int S,
-                                                   const uint32_t *__restrict__ app_idx, float *__restrict__ rgb) {
+                                                   const uint32_t *__restrict__ app_idx, int small,
+                                                   float *__restrict__ rgb) {
     extern __shared__ __align__(16) char lds[];
     using Mm = Mma<PREC>;
     using frag = typename Mm::frag;
@@ -408,46 +435,55 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
     const unsigned wpb = MlpBlock<PREC>::N / LM_WAVE;
     const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * wpb + threadIdx.x / LM_WAVE;
     const uint64_t n_waves = (uint64_t)gridDim.x * wpb;
-    // the lane's 16 input rows (features, view direction, zeros) of its sample in each column block
+    // The lane's 16 input rows (features, view direction, zeros) of its sample in each column block.  Half h
+    // holds rows row_of(v, 0) + 4 h: features up to row 23, then rows 24..26 (features, h = 0) or 28..30 (the
+    // view direction, h = 1); rows 27 and 31 are zero.  Two base addresses per lane and compile-time offsets
+    // instead of an address per load; when the feature array is below 4 GB (`small`) the bases are 32-bit
+    // byte offsets from the array's (scalar) address.
+    static_assert(row_of(0, 1) == row_of(0, 0) + 4 && row_of(11, 1) == 23 && row_of(12, 0) == 24 && row_of(12, 1) == 28 &&
+                      kAppDim == 27,
+                  "input rows per lane half");
     auto fetch = [&](uint64_t tile, float (*raw)[16]) {
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             const uint64_t p = tile * TILE + cb * 32 + j;
             const uint64_t pc = p < M ? p : M - 1;
-            const float *f = feat + pc * kAppDim;
             const float *vsrc = MODE == 0 ? view + pc * 3 : view + 6 * (size_t)(app_idx[pc] / (uint32_t)S) + 3;
-            // Half h holds rows row_of(v, 0) + 4 h: features up to row 23, then rows 24..26 (features,
-            // h = 0) or 28..30 (the view direction, h = 1); rows 27 and 31 are zero.  Two base
-            // addresses per lane and compile-time offsets instead of an address per load.
-            static_assert(row_of(0, 1) == row_of(0, 0) + 4 && row_of(11, 1) == 23 && row_of(12, 0) == 24 &&
-                              row_of(12, 1) == 28 && kAppDim == 27,
-                          "input rows per lane half");
-            const float *body = f + 4 * h;
-            const float *tail = h ? vsrc : f + 24;
+            if (small) {
+                const char *base = reinterpret_cast<const char *>(feat);
+                const uint32_t body = (uint32_t)pc * (uint32_t)(kAppDim * sizeof(float)) + 16u * h;
 #pragma unroll
-            for (int v = 0; v < 12; ++v) raw[cb][v] = body[row_of(v, 0)];
+                for (int v = 0; v < 12; ++v) raw[cb][v] = *reinterpret_cast<const float *>(base + body + 4 * row_of(v, 0));
+                if (h) {
 #pragma unroll
-            for (int v = 12; v < 15; ++v) raw[cb][v] = tail[v - 12];
+                    for (int v = 12; v < 15; ++v) raw[cb][v] = vsrc[v - 12];
+                } else {
+#pragma unroll
+                    for (int v = 12; v < 15; ++v) raw[cb][v] = *reinterpret_cast<const float *>(base + body + 4 * (12 + v));
+                }
+            } else {
+                const float *f = feat + pc * kAppDim;
+                const float *body = f + 4 * h;
+                const float *tail = h ? vsrc : f + 24;
+#pragma unroll
+                for (int v = 0; v < 12; ++v) raw[cb][v] = body[row_of(v, 0)];
+#pragma unroll
+                for (int v = 12; v < 15; ++v) raw[cb][v] = tail[v - 12];
+            }
             raw[cb][15] = 0.0f;
         }
     };
-    // the next tile's inputs travel while this tile is multiplied
-    constexpr bool kPrefetch = PREC != LM_MLP_F16X2 || LM_MLPX2_PREFETCH;
-    float nxt[NCB][16];
-    if (kPrefetch && wave_id < n_tiles) fetch(wave_id, nxt);
+    // A tile's inputs are encoded into the first layer's fragments first; the registers that held them then
+    // receive the next tile's inputs, which travel while this tile is multiplied.
+    constexpr int T1 = kSlots1 / Mm::G;
+    float raw[NCB][16];
+    if (wave_id < n_tiles) fetch(wave_id, raw);
     for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
-        float raw[NCB][16];
-        if (kPrefetch) {
-#pragma unroll
-            for (int cb = 0; cb < NCB; ++cb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) raw[cb][v] = nxt[cb][v];
-            if (tile + n_waves < n_tiles) fetch(tile + n_waves, nxt);
-        } else {
-            fetch(tile, raw);
-        }
+        frag bfrag[NCB][T1][Mm::NP];
+        encode_inputs<PREC, NCB>(raw, bfrag);
+        if (tile + n_waves < n_tiles) fetch(tile + n_waves, raw);
         float out[NCB][3];
-        colour_network<PREC, NCB>(w1, w2, w3, b1, b2, b3, raw, lane, out);
+        colour_layers<PREC, NCB>(w1, w2, w3, b1, b2, b3, bfrag, lane, out);
 #pragma unroll
         for (int cb = 0; cb < NCB; ++cb) {
             const uint64_t p = tile * TILE + cb * 32 + j;
@@ -517,6 +553,9 @@ int launch_mlp(const void *packed, int K, const float *feat, const float *view, 
                uint32_t cap, int S, const uint32_t *app_idx, float *rgb, unsigned grid, hipStream_t stream) {
     const PackLayout L = pack_layout(PREC, K);
     const size_t lds = LdsPlan<PREC>::kBytes;
+    // rows the launch can touch: the feature array stays below 4 GB when they number fewer than 2^32 / 108
+    const uint64_t rows = MODE == 0 ? M : (uint64_t)cap;
+    const int small = rows * (kAppDim * sizeof(float)) < (1ull << 32) ? 1 : 0;
     static thread_local bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mlp<PREC, MODE>),
@@ -525,7 +564,7 @@ int launch_mlp(const void *packed, int K, const float *feat, const float *view, 
         configured = true;
     }
     hipLaunchKernelGGL((k_mlp<PREC, MODE>), dim3(grid), dim3(MlpBlock<PREC>::N), lds, stream, (const char *)packed, L, feat, view,
-                       M, count, cap, S, app_idx, rgb);
+                       M, count, cap, S, app_idx, small, rgb);
     LM_CHECK_LAUNCH("k_mlp");
     return LM_OK;
 }

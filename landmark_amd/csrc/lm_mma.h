@@ -71,14 +71,28 @@ template <> struct Mma<LM_MLP_F16X2> {
     __device__ static __forceinline__ floatx16 mma(frag a, frag b, floatx16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
-    // x = hi + lo with hi = fp16(x), lo = fp16(x - hi); x - hi is exact in fp32
+    // x = hi + lo with hi = fp16(x), lo = fp16(x - hi); x - hi is exact in fp32.  Two values per register:
+    // one packed conversion gives the hi pair, and one mixed-precision fma per value (the fp16 half of hi as
+    // an operand, the result rounded to fp16 into the low or the high half) gives lo: three instructions per
+    // pair instead of the seven the compiler makes of the scalar expression (convert, convert back, subtract,
+    // convert, per value, plus packing).
     __device__ static __forceinline__ void pack(const float *s, frag *o) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u4 hi, lo;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const _Float16 hi = (_Float16)s[i];
-            o[0][i] = hi;
-            o[1][i] = (_Float16)(s[i] - (float)hi);
+        for (int i = 0; i < 4; ++i) {
+            half2v h;
+            h[0] = (_Float16)s[2 * i];
+            h[1] = (_Float16)s[2 * i + 1];
+            const uint32_t hb = __builtin_bit_cast(uint32_t, h);
+            uint32_t l;
+            asm("v_fma_mixlo_f16 %0, %1, -1.0, %2 op_sel_hi:[1,0,0]" : "=v"(l) : "v"(hb), "v"(s[2 * i]));
+            asm("v_fma_mixhi_f16 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(l) : "v"(hb), "v"(s[2 * i + 1]));
+            hi[i] = hb;
+            lo[i] = l;
         }
+        o[0] = __builtin_bit_cast(half8, hi);
+        o[1] = __builtin_bit_cast(half8, lo);
     }
 };
 
