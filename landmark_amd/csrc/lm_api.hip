@@ -89,13 +89,14 @@ int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream);
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *n_active, uint32_t *n_valid, float *acc, float *depth,
                          uint32_t *app_cnt, uint32_t *p_end, uint32_t row, uint32_t cap_valid, uint32_t *overflow,
-                         hipStream_t st);
-int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
+                         uint64_t *word_mask, hipStream_t st);
+int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const uint64_t *word_mask,
+                        const float *w_valid,
                         float weight_thres, uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
                         uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, uint32_t cap_app,
                         uint32_t *overflow, hipStream_t stream);
 int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
-                    const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid, float *acc,
+                    const uint64_t *word_mask, const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid, float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st);
 int lm_launch_basis(int prec, const void *packed, int K, const float *products, uint64_t M, const uint32_t *count,
                     uint32_t cap, float *feat, hipStream_t st);
@@ -108,6 +109,7 @@ struct Workspace {
     uint32_t *app_cnt;
     uint32_t *p_first;
     uint32_t *p_end;
+    uint64_t *word_mask;  // per ray: which of its bitmap words hold valid samples (sample counts other than 64, 128)
     uint32_t *ray_list;
     uint32_t *app_idx;
     float *app_w;
@@ -144,6 +146,7 @@ Workspace carve(char *base, int64_t N, int32_t S, int32_t K, bool need_products,
     w.app_cnt = (uint32_t *)take((uint64_t)N * 4);
     w.p_first = (uint32_t *)take((uint64_t)N * 4);
     w.p_end = (uint32_t *)take((uint64_t)N * 4);
+    w.word_mask = (uint64_t *)take((uint64_t)N * 8);
     w.ray_list = (uint32_t *)take((uint64_t)N * 4 * LM_RAY_BINS);  // one list per bin of the marching queue
     w.app_idx = (uint32_t *)take(cap * 4);
     w.app_w = (float *)take(cap * 4);
@@ -265,14 +268,17 @@ int render_chunk(const lm_model *m, int K, const float *rays, int64_t N, void *w
     if (int rc = lm_launch_zero_counters(cnt, st)) return rc;
     if (int rc = lm_launch_cull_setup(&m->geom, rays, N, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS,
                                       cnt + LM_STAT_N_VALID, w.acc, depth_map, w.app_cnt, w.p_end, row, (uint32_t)w.cap_valid,
-                                      cnt + LM_STAT_OVERFLOW, st))
+                                      cnt + LM_STAT_OVERFLOW, w.word_mask, st))
         return rc;
     mark(LM_STAGE_CULL);
-    if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, w.ray_list, cnt + LM_STAT_BINS, (uint32_t)N, cnt + LM_STAT_QUEUE,
+    // the cull writes word masks for rays of three bitmap words and more (other sample counts take the kernel
+    // with one lane per word, whose rays have one or two words)
+    const uint64_t *masks = (S == 64 || S == 128) ? nullptr : w.word_mask;
+    if (int rc = lm_launch_march(m, rays, w.bitmap, w.p_first, masks, w.ray_list, cnt + LM_STAT_BINS, (uint32_t)N, cnt + LM_STAT_QUEUE,
                                  w.w_valid, w.acc, depth_map, w.app_cnt, w.p_end, cnt + LM_STAT_N_MARCHED, st))
         return rc;
     mark(LM_STAGE_DENSITY);
-    if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.p_first, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
+    if (int rc = lm_launch_app_slots(S, N, w.bitmap, w.p_first, masks, w.w_valid, m->weight_thres, w.app_cnt, w.p_end,
                                      w.app_first, w.app_idx, w.app_w, cnt + LM_STAT_N_APP, row, (uint32_t)w.cap_app,
                                      cnt + LM_STAT_OVERFLOW, st))
         return rc;

@@ -285,31 +285,52 @@ __device__ __forceinline__ uint32_t lm_ray_order(uint32_t o, uint32_t N, uint32_
 }
 
 // Iterates the set bits of the sample bitmap in [flat0, flat1): the valid samples of one ray.
-struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
+// With a word mask (bit i set = the ray has valid samples in its i-th bitmap word, written by the cull of
+// the whole-chunk render for rays of up to 64 words) the walk jumps from one non-empty word to the next and
+// asks for the word after it at once, so that a long, mostly empty ray costs one memory round trip per
+// non-empty word, overlapped with the work on the previous one, instead of one per word.
+struct BitWalk {
     const uint64_t *bitmap;
     const uint32_t *prefix;
-    uint64_t w, w_last, bits, flat1;
+    uint64_t w, w0, w_last, bits, flat1;
+    uint64_t todo, ahead;  // masked walk: words still to visit (relative to w0), the next one's content
     uint32_t pos;
+    bool masked;
     __device__ __forceinline__ void start(const uint64_t *bm, const uint32_t *pf, uint64_t flat0, uint64_t flat1_) {
-        bitmap = bm; prefix = pf; flat1 = flat1_;
-        w = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
+        bitmap = bm; prefix = pf; flat1 = flat1_; masked = false; todo = 0; ahead = 0;
+        w = w0 = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
         const uint64_t raw = bm[w];
         const unsigned b0 = (unsigned)(flat0 & 63);
         const uint64_t below = b0 ? ((1ull << b0) - 1ull) : 0ull;
         pos = pf[w] + (uint32_t)__popcll(raw & below);
-        bits = mask_tail(raw & ~below);
+        bits = mask_tail(raw & ~below, w);
     }
-    // same walk when the compact position of the first sample is known (a per-ray table)
-    __device__ __forceinline__ void start_at(const uint64_t *bm, uint64_t flat0, uint64_t flat1_, uint32_t pos0) {
+    // same walk when the compact position of the first sample is known (a per-ray table); `mask` as above,
+    // ~0 when not known
+    __device__ __forceinline__ void start_at(const uint64_t *bm, uint64_t flat0, uint64_t flat1_, uint32_t pos0,
+                                             uint64_t mask = ~0ull) {
         bitmap = bm; prefix = nullptr; flat1 = flat1_;
-        w = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
+        w = w0 = flat0 >> 6; w_last = (flat1_ - 1) >> 6;
         const unsigned b0 = (unsigned)(flat0 & 63);
         const uint64_t below = b0 ? ((1ull << b0) - 1ull) : 0ull;
         pos = pos0;
-        bits = mask_tail(bm[w] & ~below);
+        masked = mask != ~0ull && w_last - w0 < 64;
+        if (!masked) {
+            todo = 0; ahead = 0;
+            bits = mask_tail(bm[w] & ~below, w);
+            return;
+        }
+        todo = mask;
+        bits = 0;
+        if (todo & 1ull) bits = mask_tail(bm[w0] & ~below, w0);
+        todo &= ~1ull;
+        fetch_ahead();
     }
-    __device__ __forceinline__ uint64_t mask_tail(uint64_t x) const {
-        if (w == w_last) {
+    __device__ __forceinline__ void fetch_ahead() {
+        if (todo) ahead = bitmap[w0 + (uint64_t)(__ffsll((unsigned long long)todo) - 1)];
+    }
+    __device__ __forceinline__ uint64_t mask_tail(uint64_t x, uint64_t at) const {
+        if (at == w_last) {
             const unsigned e = (unsigned)(flat1 & 63);
             if (e) x &= (1ull << e) - 1ull;
         }
@@ -318,9 +339,17 @@ struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
     // next set bit -> flat index; false when exhausted.  `pos` is the compact position of it.
     __device__ __forceinline__ bool next(uint64_t &flat) {
         while (bits == 0) {
-            if (w == w_last) return false;
-            ++w;
-            bits = mask_tail(bitmap[w]);
+            if (masked) {
+                if (todo == 0) return false;
+                w = w0 + (uint64_t)(__ffsll((unsigned long long)todo) - 1);
+                todo &= todo - 1;
+                bits = mask_tail(ahead, w);
+                fetch_ahead();
+            } else {
+                if (w == w_last) return false;
+                ++w;
+                bits = mask_tail(bitmap[w], w);
+            }
         }
         const int b = __ffsll((unsigned long long)bits) - 1;
         bits &= bits - 1;
@@ -328,4 +357,3 @@ struct BitWalk {  // iterates the set bits of bitmap in [flat0, flat1)
         return true;
     }
 };
-

@@ -115,17 +115,18 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
     const uint64_t r = lm_ray_order((uint32_t)o, (uint32_t)N, row);
     float c0 = 0.0f, c1 = 0.0f, c2 = 0.0f;
     const uint32_t first = app_first[r], n = app_cnt[r];
-    // four slots per trip, all sixteen loads issued before the sums (which stay in slot order)
-    for (uint32_t i = 0; i < n; i += 4) {
-        float w[4], c[4][3];
+    // eight slots per trip, all loads issued before the sums (which stay in slot order)
+    constexpr int kBatch = 8;
+    for (uint32_t i = 0; i < n; i += kBatch) {
+        float w[kBatch], c[kBatch][3];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kBatch; ++u) {
             const uint32_t s = first + (i + u < n ? i + u : n - 1);
             w[u] = app_w[s];
             c[u][0] = rgb[3 * (size_t)s]; c[u][1] = rgb[3 * (size_t)s + 1]; c[u][2] = rgb[3 * (size_t)s + 2];
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < kBatch; ++u)
             if (i + u < n) {
                 c0 = fmaf(w[u], c[u][0], c0); c1 = fmaf(w[u], c[u][1], c1); c2 = fmaf(w[u], c[u][2], c2);
             }
@@ -143,6 +144,7 @@ __global__ __launch_bounds__(kBlock) void k_composite(uint64_t N, const uint32_t
 // atomic), filled in sample order from the weights of the ray's samples [first, p_end).
 __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const uint64_t *__restrict__ bitmap,
                                                       const uint32_t *__restrict__ p_first,
+                                                      const uint64_t *__restrict__ word_mask,
                                                       const float *__restrict__ w_valid, float weight_thres,
                                                       uint32_t *__restrict__ app_cnt,
                                                       const uint32_t *__restrict__ p_end,
@@ -176,16 +178,17 @@ __global__ __launch_bounds__(kBlock) void k_app_slots(int S, uint64_t N, const u
         for (uint32_t i = slot; i < cap_app && i < slot + cnt; ++i) { app_idx[i] = (uint32_t)(r * (uint64_t)S); app_w[i] = 0.0f; }
     } else if (cnt) {
         BitWalk it;
-        it.start_at(bitmap, r * (uint64_t)S, (r + 1) * (uint64_t)S, p_first[r]);
+        it.start_at(bitmap, r * (uint64_t)S, (r + 1) * (uint64_t)S, p_first[r], word_mask ? word_mask[r] : ~0ull);
         const uint32_t end = p_end[r];
         uint64_t flat;
-        // four weights per trip so that their loads overlap; the walk over the bitmap stays in order
-        for (uint32_t p = it.pos; p < end; p += 4) {
-            float wgt[4];
+        // eight weights per trip so that their loads overlap; the walk over the bitmap stays in order
+        constexpr int kBatch = 8;
+        for (uint32_t p = it.pos; p < end; p += kBatch) {
+            float wgt[kBatch];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) wgt[u] = w_valid[p + u < end ? p + u : end - 1];
+            for (int u = 0; u < kBatch; ++u) wgt[u] = w_valid[p + u < end ? p + u : end - 1];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kBatch; ++u) {
                 if (p + u >= end) break;
                 it.next(flat);
                 if (wgt[u] > weight_thres) {
@@ -250,12 +253,13 @@ int lm_launch_zero_counters(uint32_t *counters, hipStream_t stream) {
     return LM_OK;
 }
 
-int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const float *w_valid,
+int lm_launch_app_slots(int S, int64_t N, const uint64_t *bitmap, const uint32_t *p_first, const uint64_t *word_mask,
+                        const float *w_valid,
                         float weight_thres, uint32_t *app_cnt, const uint32_t *p_end, uint32_t *app_first,
                         uint32_t *app_idx, float *app_w, uint32_t *app_count, uint32_t row, uint32_t cap_app,
                         uint32_t *overflow, hipStream_t stream) {
     const unsigned grid = (unsigned)(((uint64_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, p_first, w_valid,
+    hipLaunchKernelGGL(k_app_slots, dim3(grid), dim3(kBlock), 0, stream, S, (uint64_t)N, bitmap, p_first, word_mask, w_valid,
                        weight_thres, app_cnt, p_end, app_first, app_idx, app_w, app_count, row, cap_app, overflow);
     LM_CHECK_LAUNCH("k_app_slots");
     return LM_OK;

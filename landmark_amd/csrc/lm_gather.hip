@@ -17,11 +17,20 @@
 #include "lm_common.h"
 #include "lm_mma.h"
 
+#ifndef LM_MARCH_NS
+#define LM_MARCH_NS 4
+#endif
+// chunks of up to this many rays march with a wave per ray (too few rays to fill the GPU with a quad each)
+#ifndef LM_WAVE_MARCH_RAYS
+#define LM_WAVE_MARCH_RAYS 16384
+#endif
+
 namespace {
 
 constexpr int kBlock = 256;
 constexpr int kQuad = 4;
 constexpr int kTile = kBlock / kQuad;  // samples per workgroup iteration
+constexpr uint32_t kWaveMarchRays = LM_WAVE_MARCH_RAYS;
 
 struct PlaneSet {
     lm_plane p[LM_MAX_PLANES];
@@ -514,6 +523,7 @@ template <typename T, int NS>  // NS samples of a ray per round
 __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
                                                   const float *__restrict__ rays, const uint64_t *__restrict__ bitmap,
                                                   const uint32_t *__restrict__ p_first,
+                                                  const uint64_t *__restrict__ word_mask,
                                                   const uint32_t *__restrict__ ray_list,
                                                   const uint32_t *__restrict__ bins, uint32_t n_rays,
                                                   uint32_t *__restrict__ queue,
@@ -541,7 +551,8 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
     uint64_t flat0 = 0;
     float ray[6] = {0, 0, 0, 0, 0, 0}, rp = 0.0f, Tr = 1.0f, acc = 0.0f, depth = 0.0f;
     BitWalk it;
-    it.bits = 0; it.w = it.w_last = 0; it.flat1 = 0; it.pos = 0; it.bitmap = bitmap; it.prefix = nullptr;
+    it.bits = 0; it.w = it.w0 = it.w_last = 0; it.flat1 = 0; it.pos = 0; it.bitmap = bitmap; it.prefix = nullptr;
+    it.todo = it.ahead = 0; it.masked = false;
     while (true) {
         // quads without a ray take the next ones from the queue: one atomic per wave and round
         const bool need = !have && !done;
@@ -566,7 +577,7 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
                     ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
                     rp = lm_ray_param(g, ray);
                     flat0 = (uint64_t)r * (uint64_t)S;
-                    it.start_at(bitmap, flat0, flat0 + S, p_first[r]);
+                    it.start_at(bitmap, flat0, flat0 + S, p_first[r], word_mask ? word_mask[r] : ~0ull);
                     p = it.pos;
                     Tr = 1.0f; acc = 0.0f; depth = 0.0f; cnt = 0;
                     have = true;
@@ -643,6 +654,122 @@ __global__ __launch_bounds__(kBlock) void k_march(lm_geom g, PlaneSet ps, const 
     if (qlane != 0) marched = 0;
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) marched += __shfl_xor(marched, d);
+    if (lane == 0 && marched) atomicAdd(n_marched, marched);
+}
+
+// ---- the same march with a whole wave per ray ------------------------------------------------
+// For chunks with too few rays to fill the GPU with one quad each (a caller that keeps the reference's chunks
+// of a few thousand rays), and for their long rays: a launch of the kernel above lasts as long as the longest
+// chain of dependent gathers, four samples per round.  Here a wave owns a ray and takes one 64-sample word of
+// its bitmap per round: lane j prepares sample j of the word, quad i gathers samples 4i .. 4i+3 (the same
+// density_sum_n, quads without a valid sample sit the round out), so a round's 64 densities come back in one
+// memory round trip.  The transmittance then runs through the word's valid samples in order, every lane
+// computing the same scalars from values read off the owning lanes: the same operations in the same order as
+// the quad march, hence the same bits (weights, sums, counts, the sample at which a ray stops), whichever of
+// the two kernels a chunk's size selects.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void k_march_wave(lm_geom g, PlaneSet ps, const float *__restrict__ den_w,
+                                                       const float *__restrict__ rays, const uint64_t *__restrict__ bitmap,
+                                                       const uint32_t *__restrict__ p_first,
+                                                       const uint64_t *__restrict__ word_mask,
+                                                       const uint32_t *__restrict__ ray_list,
+                                                       const uint32_t *__restrict__ bins, uint32_t n_rays, int act,
+                                                       float shift, float distance_scale, float weight_thres, float term_eps,
+                                                       float *__restrict__ w_valid, float *__restrict__ acc_out,
+                                                       float *__restrict__ depth_out, uint32_t *__restrict__ app_cnt,
+                                                       uint32_t *__restrict__ p_end_out, uint32_t *__restrict__ n_marched) {
+    const unsigned lane = lm_lane(), qlane = lane & 3u;
+    const uint32_t end0 = bins[0], end1 = end0 + bins[1], end2 = end1 + bins[2], n_active = end2 + bins[3];
+    const uint32_t n_waves = gridDim.x * (kBlock / LM_WAVE);
+    const int S = g.S;
+    uint32_t marched = 0;
+    // everything that steers a wave is the same on all of its lanes: kept in scalar registers
+    auto uniform = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+    auto uniform64 = [&](uint64_t v) { return ((uint64_t)uniform((uint32_t)(v >> 32)) << 32) | uniform((uint32_t)v); };
+    for (uint32_t idx = uniform(blockIdx.x * (kBlock / LM_WAVE) + threadIdx.x / LM_WAVE); idx < n_active; idx += n_waves) {
+        const uint32_t r = idx < end0   ? ray_list[idx]
+                           : idx < end1 ? ray_list[(size_t)n_rays + (idx - end0)]
+                           : idx < end2 ? ray_list[2 * (size_t)n_rays + (idx - end1)]
+                                        : ray_list[3 * (size_t)n_rays + (idx - end2)];
+        float ray[6];
+        {
+            const float2 *rp2 = reinterpret_cast<const float2 *>(rays + 6 * (size_t)r);
+            const float2 a = rp2[0], b = rp2[1], c = rp2[2];
+            ray[0] = a.x; ray[1] = a.y; ray[2] = b.x; ray[3] = b.y; ray[4] = c.x; ray[5] = c.y;
+        }
+        const float rp = lm_ray_param(g, ray);
+        const uint64_t flat0 = (uint64_t)r * (uint64_t)S, flat1 = flat0 + (uint64_t)S;
+        const uint64_t w0 = flat0 >> 6, w_last = (flat1 - 1) >> 6;
+        uint64_t todo = word_mask ? uniform64(word_mask[r]) : ~0ull;  // the ray's non-empty words; all ones: every word
+        const bool masked = todo != ~0ull && w_last - w0 < 64;
+        uint32_t p = uniform(p_first[r]), cnt = 0;
+        float Tr = 1.0f, acc = 0.0f, depth = 0.0f;
+        bool finish = false;
+        for (uint64_t w = w0; !finish;) {
+            if (masked) {
+                if (todo == 0) break;
+                w = w0 + (uint64_t)(__ffsll((unsigned long long)todo) - 1);
+                todo &= todo - 1;
+            } else if (w > w_last) {
+                break;
+            }
+            uint64_t bits = uniform64(bitmap[w]);
+            if (w == w0 && (flat0 & 63)) bits &= ~((1ull << (flat0 & 63)) - 1ull);  // a neighbouring ray's samples share the word
+            if (w == w_last && (flat1 & 63)) bits &= (1ull << (flat1 & 63)) - 1ull;
+            if (bits) {
+                // lane j prepares sample j of the word; samples that are not valid get the coordinates of the word's
+                // first valid one (in range for the tables, results unused)
+                const bool mine = (bits >> lane) & 1ull;
+                const int j_m = mine ? (int)lane : __ffsll((unsigned long long)bits) - 1;
+                const int s_m = (int)(w * 64 + (uint64_t)j_m - flat0);
+                const float z_m = lm_sample_z(g, rp, s_m);
+                float alpha_m = 0.0f;
+                if ((bits >> (lane & ~3u)) & 0xFull) {  // the quad has a valid sample
+                    float q_m[4], f[4];
+                    {
+                        float pt[3];
+                        lm_point(ray, z_m, pt);
+                        lm_normalise(g, pt, q_m);
+                        q_m[3] = __int_as_float(g.div0 > 0 ? lm_block_coords(g, q_m) : 0);
+                    }
+                    density_sum_n<T, 4>(ps, q_m, qlane, den_w, f);
+                    float f_m = f[0];
+#pragma unroll
+                    for (int n = 1; n < 4; ++n)
+                        if ((int)qlane == n) f_m = f[n];
+                    const float sig = activate(f_m, act, shift);
+                    const float dist = (s_m + 1 < S) ? lm_sample_z(g, rp, s_m + 1) - z_m : 0.0f;
+                    const float d2 = dist * distance_scale;
+                    alpha_m = 1.0f - expf(-sig * d2);
+                }
+                marched += (uint32_t)__popcll(bits);
+                // the word's valid samples in order; every lane carries the same transmittance and sums
+                float w_mine = 0.0f;
+                uint32_t done = 0;
+                for (uint64_t rem = bits; rem;) {
+                    const int j = __ffsll((unsigned long long)rem) - 1;
+                    rem &= rem - 1;
+                    const float alpha = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(alpha_m), j));
+                    const float z = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(z_m), j));
+                    const float wgt = alpha * Tr;
+                    Tr = Tr * ((1.0f - alpha) + 1e-10f);
+                    if ((int)lane == j) w_mine = wgt;
+                    acc += wgt;
+                    depth += wgt * z;
+                    cnt += wgt > weight_thres;
+                    ++done;
+                    if (term_eps > 0.0f && Tr < term_eps) { finish = true; break; }
+                }
+                const uint32_t rank = lm_mbcnt(bits);
+                if (mine && rank < done) w_valid[p + rank] = w_mine;
+                p += done;
+            }
+            ++w;
+        }
+        if (lane == 0) {
+            acc_out[r] = acc; depth_out[r] = depth; app_cnt[r] = cnt; p_end_out[r] = p;
+        }
+    }
     if (lane == 0 && marched) atomicAdd(n_marched, marched);
 }
 
@@ -1036,7 +1163,7 @@ int lm_launch_app_features(const lm_model *m, const float *rays, const uint32_t 
 
 // Density + transmittance march over the rays listed in ray_list (those with valid samples).
 int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap, const uint32_t *p_first,
-                    const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid,
+                    const uint64_t *word_mask, const uint32_t *ray_list, const uint32_t *bins, uint32_t n_rays, uint32_t *queue, float *w_valid,
                     float *acc,
                     float *depth, uint32_t *app_cnt, uint32_t *p_end, uint32_t *n_marched, hipStream_t st) {
     int dtype;
@@ -1059,16 +1186,34 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     };
     int c_max = 0;
     for (int k = 0; k < m->n_planes; ++k) c_max = std::max(c_max, (int)m->density[k].C);
+    if (n_rays <= kWaveMarchRays) {
+        // few rays: a wave per ray, one launch-wide round trip per 64-sample word instead of one per four samples
+        const unsigned grid = std::min<unsigned>((n_rays + kBlock / LM_WAVE - 1) / (kBlock / LM_WAVE), (unsigned)lm_persistent_blocks(8));
+#define LM_MARCH_WAVE(T_)                                                                                             \
+    hipLaunchKernelGGL((k_march_wave<T_>), dim3(grid), dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap, \
+                       p_first, word_mask, ray_list, bins, n_rays, m->act, m->density_shift, m->distance_scale,          \
+                       m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched)
+        if (dtype == LM_F32) {
+            LM_MARCH_WAVE(float);
+        } else if (c_max <= 16) {
+            LM_MARCH_WAVE(Half4);
+        } else {
+            LM_MARCH_WAVE(__half);
+        }
+#undef LM_MARCH_WAVE
+        LM_CHECK_LAUNCH("k_march_wave");
+        return LM_OK;
+    }
 #define LM_MARCH(T_, NS_)                                                                                              \
     hipLaunchKernelGGL((k_march<T_, NS_>), dim3(resident_grid(reinterpret_cast<const void *>(&k_march<T_, NS_>))),         \
                        dim3(kBlock), 0, st, m->geom, ps, m->density_basis, rays, bitmap,   \
-                       p_first, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,            \
+                       p_first, word_mask, ray_list, bins, n_rays, queue, m->act, m->density_shift, m->distance_scale,            \
                        m->weight_thres, m->term_eps, w_valid, acc, depth, app_cnt, p_end, n_marched)
     // Four samples per round: one per lane of the quad for the footprint arithmetic, 24 loads per lane and plane
     // in flight, half as many dependent round trips per ray as with two (1080p frame, nine fp32 planes: 2.70 ->
     // 2.50 ms although the kernel then holds 223 registers and two waves per SIMD instead of three).
     if (dtype == LM_F32) {
-        LM_MARCH(float, 4);
+        LM_MARCH(float, LM_MARCH_NS);
     } else if (c_max <= 16) {  // 16-byte loads would leave half of every quad idle
         LM_MARCH(Half4, 4);
     } else {

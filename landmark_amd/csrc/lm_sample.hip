@@ -221,12 +221,14 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
                                                                    uint32_t *__restrict__ n_valid, float *__restrict__ acc,
                                                                    float *__restrict__ depth, uint32_t *__restrict__ app_cnt,
                                                                    uint32_t *__restrict__ p_end, uint32_t cap_valid,
-                                                                   uint32_t *__restrict__ overflow) {
+                                                                   uint32_t *__restrict__ overflow,
+                                                                   uint64_t *__restrict__ word_mask) {
     const unsigned lane = lm_lane();
     const unsigned sub = threadIdx.x % LPR;  // this lane's share of its ray's words
     const uint64_t o = ((uint64_t)blockIdx.x * kBlock + threadIdx.x) / LPR;  // position in the visiting order
     const uint64_t r = o < N ? lm_ray_order((uint32_t)o, N, row) : o;
     uint32_t cnt = 0;
+    uint64_t words = 0;  // bit i: the ray has valid samples in its i-th bitmap word (rays of up to 64 words)
     if (r < N) {
         float ray[6];
         load_ray(rays, r, ray);
@@ -240,11 +242,16 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
             if (hi - lo == 64) bitmap[w] = bits;
             else if (bits) atomicOr(reinterpret_cast<unsigned long long *>(bitmap + w), (unsigned long long)bits);
             cnt += (uint32_t)__popcll(bits);
+            if (bits) words |= 1ull << ((w - (flat0 >> 6)) & 63u);
         }
     }
     // the ray's count on all of its lanes; its first lane speaks for it from here on
 #pragma unroll
-    for (int d = 1; d < LPR; d <<= 1) cnt += __shfl_xor(cnt, d);
+    for (int d = 1; d < LPR; d <<= 1) {
+        cnt += __shfl_xor(cnt, d);
+        const uint32_t lo = __shfl_xor((uint32_t)words, d), hi = __shfl_xor((uint32_t)(words >> 32), d);
+        words |= ((uint64_t)hi << 32) | lo;
+    }
     uint32_t incl = sub == 0 ? cnt : 0;
 #pragma unroll
     for (int d = 1; d < LM_WAVE; d <<= 1) {
@@ -262,6 +269,8 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
     const bool any = lm_ray_fits(mine ? cnt : 0u, first, cap_valid, overflow);
     if (mine) {
         p_first[r] = first;
+        // a ray of more than 64 words cannot be described: all ones = "walk every word"
+        word_mask[r] = (((r + 1) * (uint64_t)g.S - 1) >> 6) - ((r * (uint64_t)g.S) >> 6) < 64 ? words : ~0ull;
         if (!any) { acc[r] = 0.0f; depth[r] = 0.0f; app_cnt[r] = 0; p_end[r] = first; }
     }
     lm_ray_enqueue(any && mine, lm_ray_bin(cnt), (uint32_t)r, ray_list, N, bins);
@@ -513,7 +522,7 @@ extern "C" int lm_alpha_mask_pool(const float *alpha, int32_t gx, int32_t gy, in
 int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint64_t *bitmap, uint32_t *p_first,
                          uint32_t *ray_list, uint32_t *bins, uint32_t *n_valid, float *acc, float *depth,
                          uint32_t *app_cnt, uint32_t *p_end, uint32_t row, uint32_t cap_valid, uint32_t *overflow,
-                         hipStream_t st) {
+                         uint64_t *word_mask, hipStream_t st) {
     const int wpr = geom->S % 64 == 0 ? geom->S / 64 : 0;
     LM_REQUIRE((reinterpret_cast<uintptr_t>(rays) & 7u) == 0, "rays must be 8-byte aligned");
 #define LM_CULL_SETUP(W_)                                                                                             \
@@ -537,7 +546,7 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
 #define LM_CULL_SERIAL(L_)                                                                                           \
     hipLaunchKernelGGL(k_cull_rays_setup_serial<L_>, dim3((unsigned)(((uint64_t)N * L_ + kBlock - 1) / kBlock)),         \
                        dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, \
-                       depth, app_cnt, p_end, cap_valid, overflow)
+                       depth, app_cnt, p_end, cap_valid, overflow, word_mask)
         switch (lpr) {
             case 1: LM_CULL_SERIAL(1); break;
             case 2: LM_CULL_SERIAL(2); break;

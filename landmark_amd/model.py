@@ -340,6 +340,10 @@ class GridNeRFHIP:
         if self.capacity == "worst":
             return (0, 0)
         total = int(n_rays) * int(S)
+        if total * 132 <= self.small_workspace:
+            # a small chunk: the worst case costs little memory, and without the check for an overflow
+            # consecutive calls need no host synchronisation between them
+            return (0, 0)
         per_ray_app = min(int(S), int(1.001 / self.p.rayMarch_weight_thres) + 2) if self.p.rayMarch_weight_thres > 0 else int(S)
         want_valid = max(1 << 16, int(self.samples_per_ray[0] * n_rays) + 1)
         want_app = max(1 << 14, int(self.samples_per_ray[1] * n_rays) + 1)
@@ -379,6 +383,8 @@ class GridNeRFHIP:
 
     # bytes of workspace a render may take when the library picks the chunk size itself
     workspace_budget = 24 << 30
+    # chunks whose worst-case workspace stays below this are always given the worst case
+    small_workspace = 256 << 20
 
     def preferred_chunk(self, n_rays: int, N_samples: int = -1) -> int:
         """Rays per lm_render call when the caller leaves the choice to the library: up to 2^20
@@ -446,10 +452,12 @@ class GridNeRFHIP:
         (one small copy, the call's one host synchronisation), raise the capacity to what the counters ask for and
         render the affected chunks again until none overflows.  `chunks`: (slice of the ray array, the counter
         block its render wrote).  Returns the number of repeated renders; nothing to do with capacity="worst"."""
-        if self.capacity == "worst" or not chunks:
+        S = self._samples_for(N_samples)
+        # chunks rendered on a worst-case workspace cannot have overflowed: no need to look (or to synchronise)
+        pending = [(sl, c) for sl, c in chunks if self.capacities(sl.stop - sl.start, S) != (0, 0)]
+        if not pending:
             return 0
         repeats = 0
-        pending = list(chunks)
         for _ in range(6):
             host = torch.stack([c for _, c in pending]).cpu().long() & 0xFFFFFFFF
             again = []
@@ -457,7 +465,6 @@ class GridNeRFHIP:
                 if int(row[L.LM_STAT_OVERFLOW]) == 0:
                     continue
                 n = sl.stop - sl.start
-                S = self._samples_for(N_samples)
                 caps = self.capacities(n, S)
                 valid_over = caps[0] != 0 and int(row[L.LM_STAT_N_VALID]) > caps[0]
                 self._grow_capacity(n, int(row[L.LM_STAT_N_VALID]), int(row[L.LM_STAT_N_APP]), valid_over)

@@ -545,6 +545,7 @@ def test_workspace_capacity_overflow_is_reported_and_repeatable(gpu_lib, opt, S)
     assert over == 0 and torch.equal(rgb, full["rgb_map"]) and torch.equal(dep, full["depth_map"])
     # the wrapper's adaptive sizing: starts too small, reads the counters, repeats the chunk, remembers
     a = _model(p)
+    a.small_workspace = 0  # chunks this small would otherwise get the worst case
     a.samples_per_ray = [0.2 * want["n_valid"] / N, 0.2 * want["n_app"] / N]
     assert a.capacities(N, S)[0] * 4 < want["n_valid"] * 4 and a.capacities(N, S) != (0, 0)
     out, _ = a(rays, N_samples=S)
@@ -553,6 +554,37 @@ def test_workspace_capacity_overflow_is_reported_and_repeatable(gpu_lib, opt, S)
     assert a.last_counts()["overflow"] == 0
     out2, _ = a(rays, N_samples=S)  # now sized right the first time
     assert torch.equal(out2["rgb_map"], full["rgb_map"])
+
+
+@pytest.mark.parametrize("opt,S,term,fp16,div", [(1, 128, 0.0, False, None), (1, 128, 1e-4, False, None), (0, 200, 1e-4, False, None),
+                                                  (1, 64, 0.0, True, None), (0, 330, 0.0, False, None), (1, 128, 1e-4, False, (2, 3))])
+def test_both_march_kernels_give_the_same_bits(gpu_lib, opt, S, term, fp16, div):
+    """Chunks of up to 16384 rays march with a wave per ray, larger ones with a quad per ray: the same operations in
+    the same order, so a ray's result does not depend on the size of the chunk it arrives in (early termination,
+    word masks of long rays, fp16 tables and block-stacked tables included)."""
+    from landmark_amd.render import renderer_fn
+
+    if div is None:
+        p = _scene(opt=opt, S=S, thre=0.0, step_ratio=0.2, resMode=(1, 2))
+    else:
+        p = scenes.make_params(seed=11, gridSize=(10, 9, 12), near_far=[0.5, 4.5], n_importance=S, sampling_opt=opt,
+                               density_shift=0.0, resMode=(1, 2), ndims=1, plane_division=div)
+        for t in p.density_plane:
+            t.mul_(8.0)
+    if fp16:
+        p = O.to_fp16_features(p)
+    rays = scenes.pinhole_rays(200, 150, 170.0, scenes.sphere_pose(2.5, 9)).cuda()  # 30000 rays: one quad-march chunk
+    m = _model(p, term_eps=term, mlp_precision="f16x2")
+    whole, _ = renderer_fn(rays, m, chunk=1 << 20, N_samples=S, device="cuda")
+    parts, _ = renderer_fn(rays, m, chunk=7001, N_samples=S, device="cuda", exact_chunk=True)  # five wave-march chunks
+    assert float(whole["rgb_map"].min()) < 0.9
+    assert torch.equal(whole["depth_map"], parts["depth_map"])
+    assert torch.equal(whole["rgb_map"], parts["rgb_map"])
+    ref = O.render_chunk(p, rays[:3000].cpu(), N_samples=S, return_aux=True)
+    band = ((ref["weight"] - 1e-3).abs() < 2e-7).any(-1)
+    tol = (RGB_TOL_16 if fp16 else RGB_TOL_F32) + term * 4.5
+    assert (parts["rgb_map"][:3000].cpu() - ref["rgb_map"]).abs().max(-1).values[~band].max().item() <= tol
+    assert (parts["depth_map"][:3000].cpu() - ref["depth_map"]).abs()[~band].max().item() <= tol
 
 
 @pytest.mark.parametrize("S,width", [(128, 96), (64, 40), (100, 96), (128, 50)])
