@@ -212,7 +212,9 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup(lm_geom g, const flo
 // in a less regular order this way, which costs the march a little; with one or two words per ray
 // the kernel above is the better trade.  When a chunk has too few rays to fill the GPU with one lane
 // each, LPR neighbouring lanes share a ray and take every LPR-th word of it.
-template <int LPR>
+// SEG = 64: a lane's unit of work is a bitmap word; SEG = 16: a quarter of one (chunks with so few rays that even a
+// lane per word leaves most of the GPU idle), the words are then put together with atomic ORs.
+template <int LPR, int SEG>
 __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, const float *__restrict__ rays, uint32_t N,
                                                                    uint32_t row, uint64_t *__restrict__ bitmap,
                                                                    uint32_t *__restrict__ p_first,
@@ -236,8 +238,9 @@ __global__ __launch_bounds__(kBlock) void k_cull_rays_setup_serial(lm_geom g, co
         // the ray's samples are bits [flat0, flat1) of the bitmap: whole words are stored, a first or last word
         // shared with a neighbouring ray is merged into the (zeroed) bitmap
         const uint64_t flat0 = r * (uint64_t)g.S, flat1 = flat0 + (uint64_t)g.S;
-        for (uint64_t w = (flat0 >> 6) + sub; w * 64 < flat1; w += LPR) {
-            const uint64_t lo = w * 64 > flat0 ? w * 64 : flat0, hi = (w + 1) * 64 < flat1 ? (w + 1) * 64 : flat1;
+        for (uint64_t u = flat0 / SEG + sub; u * SEG < flat1; u += LPR) {
+            const uint64_t w = u * SEG / 64;
+            const uint64_t lo = u * SEG > flat0 ? u * SEG : flat0, hi = (u + 1) * SEG < flat1 ? (u + 1) * SEG : flat1;
             const uint64_t bits = segment_bits(g, ray, rp, (int)(lo - flat0), (int)(hi - lo), (int)(lo & 63));
             if (hi - lo == 64) bitmap[w] = bits;
             else if (bits) atomicOr(reinterpret_cast<unsigned long long *>(bitmap + w), (unsigned long long)bits);
@@ -529,22 +532,35 @@ int lm_launch_cull_setup(const lm_geom *geom, const float *rays, int64_t N, uint
     hipLaunchKernelGGL(k_cull_rays_setup<W_>, dim3((unsigned)(((uint64_t)N * W_ + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, \
                        *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, depth, app_cnt, p_end,  \
                        cap_valid, overflow)
-    if (wpr == 1) {
+    // a lane per (ray, word) for 64 and 128 samples, unless the chunk has so few rays that a lane per quarter word
+    // is needed to occupy the GPU
+    const bool few = (uint64_t)N * (wpr > 0 ? wpr : 1) * 8 <= (uint64_t)lm_persistent_blocks(2) * kBlock;
+    if (wpr == 1 && !few) {
         LM_CULL_SETUP(1);
-    } else if (wpr == 2) {
+    } else if (wpr == 2 && !few) {
         LM_CULL_SETUP(2);
     } else {
-        if (wpr == 0) {
+        // one lane per ray when the chunk fills the GPU that way, otherwise 2 .. 16 lanes per ray, which share its
+        // words, or quarters of its words when there are fewer words than lanes
+        const uint64_t fill = (uint64_t)lm_persistent_blocks(2) * kBlock;
+        const int words = (geom->S + 63) / 64;
+        int lpr = 1;
+        while (lpr < 16 && 2 * lpr <= words && (uint64_t)N * lpr < fill) lpr *= 2;
+        const bool quarters = (uint64_t)N * lpr * 2 <= fill && 2 * lpr > words && lpr < 16;
+        if (quarters)
+            while (lpr < 16 && 2 * lpr <= 4 * words && (uint64_t)N * lpr < fill) lpr *= 2;
+        if (wpr == 0 || quarters) {
             const uint64_t n_words = ((uint64_t)N * (uint64_t)geom->S + 63) / 64;
             const unsigned blocks = (unsigned)std::min<uint64_t>((n_words + kBlock - 1) / kBlock, 4096);
             hipLaunchKernelGGL(k_zero_words, dim3(blocks), dim3(kBlock), 0, st, bitmap, n_words);
         }
-        // one lane per ray when the chunk fills the GPU that way, otherwise 2 .. 16 lanes per ray
-        const int words = (geom->S + 63) / 64;
-        int lpr = 1;
-        while (lpr < 16 && 2 * lpr <= words && (uint64_t)N * lpr < (uint64_t)lm_persistent_blocks(2) * kBlock) lpr *= 2;
 #define LM_CULL_SERIAL(L_)                                                                                           \
-    hipLaunchKernelGGL(k_cull_rays_setup_serial<L_>, dim3((unsigned)(((uint64_t)N * L_ + kBlock - 1) / kBlock)),         \
+    if (quarters)                                                                                                    \
+        hipLaunchKernelGGL((k_cull_rays_setup_serial<L_, 16>), dim3((unsigned)(((uint64_t)N * L_ + kBlock - 1) / kBlock)), \
+                           dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid,  \
+                           acc, depth, app_cnt, p_end, cap_valid, overflow, word_mask);                                 \
+    else                                                                                                             \
+    hipLaunchKernelGGL((k_cull_rays_setup_serial<L_, 64>), dim3((unsigned)(((uint64_t)N * L_ + kBlock - 1) / kBlock)),     \
                        dim3(kBlock), 0, st, *geom, rays, (uint32_t)N, row, bitmap, p_first, ray_list, bins, n_valid, acc, \
                        depth, app_cnt, p_end, cap_valid, overflow, word_mask)
         switch (lpr) {
