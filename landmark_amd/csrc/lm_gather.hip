@@ -22,7 +22,7 @@
 #endif
 // chunks of up to this many rays march with a wave per ray (too few rays to fill the GPU with a quad each)
 #ifndef LM_WAVE_MARCH_RAYS
-#define LM_WAVE_MARCH_RAYS 16384
+#define LM_WAVE_MARCH_RAYS 12288
 #endif
 
 namespace {

@@ -559,7 +559,7 @@ def test_workspace_capacity_overflow_is_reported_and_repeatable(gpu_lib, opt, S)
 @pytest.mark.parametrize("opt,S,term,fp16,div", [(1, 128, 0.0, False, None), (1, 128, 1e-4, False, None), (0, 200, 1e-4, False, None),
                                                   (1, 64, 0.0, True, None), (0, 330, 0.0, False, None), (1, 128, 1e-4, False, (2, 3))])
 def test_both_march_kernels_give_the_same_bits(gpu_lib, opt, S, term, fp16, div):
-    """Chunks of up to 16384 rays march with a wave per ray, larger ones with a quad per ray: the same operations in
+    """Chunks of up to 12288 rays march with a wave per ray, larger ones with a quad per ray: the same operations in
     the same order, so a ray's result does not depend on the size of the chunk it arrives in (early termination,
     word masks of long rays, fp16 tables and block-stacked tables included)."""
     from landmark_amd.render import renderer_fn
