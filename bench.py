@@ -136,7 +136,7 @@ def bench_frame(args, workload):
     term_auto = args.term_eps == "auto"
     term_eps = 1e-4 / float(p.near_far[1]) if term_auto else float(args.term_eps)
     args.term_eps = term_eps
-    model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=term_eps)
+    model = GridNeRFHIP(p, device=dev, mlp_precision=args.mlp, term_eps=term_eps, capacity=args.capacity)
     model._set_app_code(args.mlp, app_code)
     torch.cuda.synchronize()
     log(f"[bench] scene {name} built in {time.time() - t0:.1f}s; tables "
@@ -471,6 +471,8 @@ def main():
                     help="c4 (default): 1080p frame of the multi-resolution model; prod: the same frame with the reference's "
                          "production shape (one orientation, AABB sampler, embedding, density projection)")
     ap.add_argument("--step-ratio", type=float, default=0.5, help="prod: grid cells per sampling step (the reference's default)")
+    ap.add_argument("--capacity", default="adaptive", choices=["adaptive", "worst"],
+                    help="render workspace: sized from the samples per ray a first frame reports, or for the worst case")
     ap.add_argument("--no-extra", action="store_true", help="c4: skip the exact-mode and one-orientation timings after the timed region")
     ap.add_argument("--planes", type=int, default=3, help="ndims of the c4 model (3 = XY,XZ,YZ; 1 = XY only)")
     ap.add_argument("--base", type=int, default=1024, help="base plane resolution of c4 (levels x1,x2,x4)")
