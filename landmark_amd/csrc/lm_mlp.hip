@@ -41,9 +41,8 @@
 #ifndef LM_MLP_NCB
 #define LM_MLP_NCB 2
 #endif
-// split-fp16 mode: eight waves with one column block each (two waves per SIMD, so that one wave's
-// encoding and conversions run under the other's MFMAs) beat four waves with two (2.37 -> 2.15 ms
-// on 2^23 rows) although 87 registers spill
+// split-fp16 mode: eight waves with one column block each beat four waves with two (the second wave of a SIMD
+// covers the first one's waits for LDS and memory; vector and matrix instructions themselves do not overlap)
 #ifndef LM_MLPX2_THREADS
 #define LM_MLPX2_THREADS 512
 #endif
@@ -52,9 +51,6 @@
 #endif
 #ifndef LM_MLPX2_NB
 #define LM_MLPX2_NB 1  // split mode: one accumulator block at a time keeps the wave inside 256 registers
-#endif
-#ifndef LM_MLPX2_PREFETCH
-#define LM_MLPX2_PREFETCH 0  // split mode: the second wave of the SIMD hides the input load, 16 registers are worth more
 #endif
 #ifndef LM_MLP16_NB1
 #define LM_MLP16_NB1 4  // 16-bit modes with one column block: row blocks per pass
