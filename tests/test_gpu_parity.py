@@ -421,7 +421,14 @@ def test_render_configuration_sweep(gpu_lib):
             p = O.to_fp16_features(p)
         rays = scenes.pinhole_rays(w, h, 0.8 * max(w, h), scenes.sphere_pose(2.5, seed % 17))[cut:]
         try:
-            _check_render(p, rays, RGB_TOL_16 if fp16 else RGB_TOL_F32, S=S if opt == 0 else -1, mlp_precision="f16x2")
+            _, out = _check_render(p, rays, RGB_TOL_16 if fp16 else RGB_TOL_F32, S=S if opt == 0 else -1, mlp_precision="f16x2")
+            # the same rays repeated until the chunk takes the large-chunk kernels (a quad per ray in the march, a lane
+            # per word or ray in the cull) instead of the small-chunk ones: identical bits for the first copy
+            reps = 13000 // rays.shape[0] + 1
+            big, _ = _model(p, mlp_precision="f16x2")(rays.repeat(reps, 1), N_samples=S if opt == 0 else -1)
+            n = rays.shape[0]
+            assert torch.equal(big["rgb_map"][:n], out["rgb_map"]) and torch.equal(big["depth_map"][:n], out["depth_map"])
+            assert torch.equal(big["rgb_map"][-n:], out["rgb_map"])
         except AssertionError as e:
             raise AssertionError(f"configuration {it}: opt {opt} S {S} res {res} ndims {ndims} fp16 {fp16} act {act} "
                                  f"shift {shift} thre {thre} mask {mask} {w}x{h} cut {cut} seed {seed}: {e}") from e
