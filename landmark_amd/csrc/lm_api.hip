@@ -18,17 +18,20 @@ void lm_set_error(const char *fmt, ...) {
 extern "C" const char *lm_last_error(void) { return g_err; }
 extern "C" int lm_abi_version(void) { return LM_ABI_VERSION; }
 
+int lm_current_device(void) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = 0;
+    return dev < LM_MAX_DEVICES ? dev : LM_MAX_DEVICES - 1;
+}
+
 int lm_persistent_blocks(int blocks_per_cu) {
-    static thread_local int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
+    static thread_local int cus[LM_MAX_DEVICES] = {};  // per device: a thread may switch GPUs between calls
+    const int dev = lm_current_device();
+    if (cus[dev] == 0) {
+        int n = 0;
+        cus[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
     }
-    return cus * blocks_per_cu;
+    return cus[dev] * blocks_per_cu;
 }
 
 // ---- [C,H,W] -> [H,W,C] ---------------------------------------------------------------------
@@ -202,7 +205,7 @@ extern "C" int lm_render(const lm_model *m, const float *rays, int64_t N, void *
 static __device__ __align__(256) unsigned char scratch[LM_STATIC_WORKSPACE_BYTES];
 
 namespace {
-constexpr int kMaxDevices = 64;
+constexpr int kMaxDevices = LM_MAX_DEVICES;
 std::mutex g_scratch_lock;
 void *g_scratch_ptr[kMaxDevices] = {};
 

@@ -28,6 +28,10 @@ void lm_set_error(const char *fmt, ...);
 
 static inline bool lm_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Launch attributes and device facts are cached per thread and device (index of the current device, clamped)
+#define LM_MAX_DEVICES 64
+int lm_current_device(void);
+
 // Number of workgroups for grid-stride kernels: enough resident waves to cover every CU
 // several times over; 256 CUs in 8 XCDs on MI355X.
 int lm_persistent_blocks(int blocks_per_cu);

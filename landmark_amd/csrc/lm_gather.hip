@@ -938,7 +938,8 @@ int launch_app_feat(int nu, const lm_model *m, const PlaneSet &ps, int K, const 
 #define LM_AF_CASE(NU_)                                                                                            \
     case NU_: {                                                                                                    \
         auto kern = &k_app_feat<PREC, T, NU_>;                                                                     \
-        static thread_local size_t reserved = 0; /* the attribute is set once per thread, kernel and size */       \
+        static thread_local size_t reserved_on[LM_MAX_DEVICES] = {}; /* set once per thread, device, kernel, size */ \
+        size_t &reserved = reserved_on[lm_current_device()];                                                       \
         if (reserved != lds) {                                                                                     \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                               \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);              \
@@ -1173,8 +1174,11 @@ int lm_launch_march(const lm_model *m, const float *rays, const uint64_t *bitmap
     // as many workgroups as are resident at once (the kernel's register count decides), at most four per CU
     auto resident_grid = [](const void *kernel) {
         // asked once per thread and kernel: the answer depends on the kernel's registers only
-        static thread_local const void *known[4] = {nullptr, nullptr, nullptr, nullptr};
-        static thread_local unsigned grid[4] = {0, 0, 0, 0};
+        static thread_local const void *known_on[LM_MAX_DEVICES][4] = {};
+        static thread_local unsigned grid_on[LM_MAX_DEVICES][4] = {};
+        const int dev = lm_current_device();
+        const void **known = known_on[dev];
+        unsigned *grid = grid_on[dev];
         for (int i = 0; i < 4; ++i)
             if (known[i] == kernel) return grid[i];
         int per_cu = 0;

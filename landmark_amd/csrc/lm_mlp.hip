@@ -552,7 +552,8 @@ int launch_mlp(const void *packed, int K, const float *feat, const float *view, 
     // rows the launch can touch: the feature array stays below 4 GB when they number fewer than 2^32 / 108
     const uint64_t rows = MODE == 0 ? M : (uint64_t)cap;
     const int small = rows * (kAppDim * sizeof(float)) < (1ull << 32) ? 1 : 0;
-    static thread_local bool configured = false;
+    static thread_local bool configured_on[LM_MAX_DEVICES] = {};  // the attribute belongs to a device's copy of the kernel
+    bool &configured = configured_on[lm_current_device()];
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&k_mlp<PREC, MODE>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -42,6 +42,27 @@ def test_isolated_gather_full_size_closed_form(gpu_lib):
     assert err < 2e-4, err  # 192 fp32 terms of magnitude <= 1
 
 
+@pytest.mark.parametrize("prec,tol", [("f16", 4e-3), ("f16x2", 3e-6)])
+def test_isolated_colour_network_full_size(gpu_lib, prec, tol):
+    """2^23 rows (27 features ~ N(0,1), unit view directions) through the fused network: a strided sample against
+    the oracle, and row independence at full size (a reversed copy of the input gives the reversed output, bit for bit:
+    rows meet other rows in a wave tile, a different lane and a different workgroup)."""
+    dev = "cuda"
+    p = scenes.make_params(seed=3, gridSize=(8, 8, 8), density_n_comp=4, app_n_comp=48)
+    m = _model(p, mlp_precision=prec)
+    M = 1 << 23
+    g = torch.Generator(device=dev).manual_seed(3)
+    feat = torch.randn((M, 27), device=dev, generator=g)
+    view = torch.nn.functional.normalize(torch.randn((M, 3), device=dev, generator=g), dim=-1)
+    out = m.render_module(view, feat)
+    assert out.shape == (M, 3) and float(out.min()) >= 0.0 and float(out.max()) <= 1.0
+    idx = torch.arange(0, M, 127, device=dev)[: 1 << 16]
+    ref = O.mlp_render(p, view[idx].cpu(), feat[idx].cpu())
+    assert (out[idx].cpu() - ref).abs().max().item() <= tol
+    back = m.render_module(view.flip(0).contiguous(), feat.flip(0).contiguous())
+    assert torch.equal(back.flip(0), out)
+
+
 @pytest.fixture(scope="module")
 def frame():
     p = scenes.c4_scene(P=3, base=1024, device="cuda", density_shift=0.0)
