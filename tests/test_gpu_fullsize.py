@@ -63,6 +63,41 @@ def test_isolated_colour_network_full_size(gpu_lib, prec, tol):
     assert torch.equal(back.flip(0), out)
 
 
+def test_largest_chunk_the_abi_admits(gpu_lib):
+    """One lm_render call of 2^25 - 1 rays x 128 samples (N*S = 2^32 - 128, the last sample index a chunk may have):
+    a 1024 x 512 image repeated 64 times.  Every copy must equal the first bit for bit (sample and slot indices
+    near 2^32 behave like those near 0), the first must equal the same image rendered on its own, and one ray more
+    is refused."""
+    from landmark_amd import _lib as L
+    from tests.test_gpu_parity import _scene
+
+    dev = "cuda"
+    p = _scene(opt=1, S=128, grid=(33, 37, 41), step_ratio=2.0)
+    m = _model(p, mlp_precision="f16x2")
+    tile = scenes.pinhole_rays(1024, 512, 900.0, scenes.sphere_pose(2.5, 5)).to(dev)
+    T = tile.shape[0]
+    N = (1 << 25) - 1
+    rays = tile.repeat(64, 1)[:N].contiguous()
+    alone = m(tile)[0]
+    one = m.last_counts()
+    assert one["n_valid"] > T and one["n_app"] > T // 4
+    m.samples_per_ray = [1.3 * one["n_valid"] / T, 1.3 * one["n_app"] / T]
+    rgb = torch.full((N, 3), -1.0, device=dev)
+    depth = torch.full((N,), -1.0, device=dev)
+    m.render_into(rays, rgb, depth)
+    c = m.last_counts()
+    assert c["overflow"] == 0
+    assert 63 * one["n_valid"] <= c["n_valid"] <= 64 * one["n_valid"] and 63 * one["n_app"] <= c["n_app"] <= 64 * one["n_app"]
+    assert torch.equal(rgb[:T], alone["rgb_map"]) and torch.equal(depth[:T], alone["depth_map"])
+    for k in (1, 31, 62):
+        assert torch.equal(rgb[k * T:(k + 1) * T], rgb[:T]) and torch.equal(depth[k * T:(k + 1) * T], depth[:T])
+    assert torch.equal(rgb[63 * T:], rgb[:T - 1]) and torch.equal(depth[63 * T:], depth[:T - 1])
+    del rgb, depth
+    more = torch.cat([rays, tile[:1]])
+    with pytest.raises(L.LandmarkError, match="32-bit"):
+        m.render_into(more, torch.empty((N + 1, 3), device=dev), torch.empty((N + 1,), device=dev))
+
+
 @pytest.fixture(scope="module")
 def frame():
     p = scenes.c4_scene(P=3, base=1024, device="cuda", density_shift=0.0)
