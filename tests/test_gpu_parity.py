@@ -388,14 +388,27 @@ def test_render_random_scenes(gpu_lib, opt, act, shift, res, ndims):
     assert ref["app_mask"].any(), "scene must exercise the colour network"
 
 
-@pytest.mark.parametrize("opt,S", [(1, 192), (1, 320), (0, 448), (1, 100), (1, 600), (0, 1100)])
-def test_render_other_sample_counts(gpu_lib, opt, S):
+@pytest.mark.parametrize("opt,S,step", [(1, 192, 0.08), (1, 320, 0.08), (0, 448, 0.08), (1, 100, 0.08), (1, 600, 0.08),
+                                        (0, 1100, 0.08), (0, 3544, 0.004), (0, 4500, 0.0031)])
+def test_render_other_sample_counts(gpu_lib, opt, S, step):
     """Sample counts other than 64 and 128 take the cull that walks a ray's bitmap words in one lane, or, for a
-    chunk as small as this one, in 2, 4, 8 or 16 lanes (3, 5, 7, 2, 10 and 18 words per ray here)."""
-    p = _scene(opt=opt, S=S, shift=0.0, step_ratio=0.08, thre=0.0)
+    chunk as small as this one, in 2, 4, 8 or 16 lanes (3, 5, 7, 2, 10 and 18 words per ray here; 56 words at the
+    reference's default step, and 71: beyond the 64 words a ray's word mask can describe, so every word is walked).
+    The last two use a step that spreads the samples over the whole box, so that late words hold valid samples."""
+    p = _scene(opt=opt, S=S, shift=0.0, step_ratio=step, thre=0.0)
     rays = scenes.pinhole_rays(40, 40, 34.0, scenes.sphere_pose(2.5, 9))
     ref, _ = _check_render(p, rays, RGB_TOL_F32, S=S)
     assert ref["app_mask"].any()
+    if S > 1100:
+        last = ref["ray_valid"].reshape(rays.shape[0], S)[:, S - S // 4:].any()
+        assert last, "valid samples in the last quarter of the rays"
+    if S > 1100:
+        # the same rays often enough for the quad-per-ray march (chunks above 12 288 rays)
+        m = _model(p, mlp_precision="f16x2")
+        small = m(rays, N_samples=S)[0]
+        many = m(rays.repeat(8, 1), N_samples=S)[0]
+        assert torch.equal(many["rgb_map"][-rays.shape[0]:], small["rgb_map"])
+        assert torch.equal(many["depth_map"][-rays.shape[0]:], small["depth_map"])
 
 
 def test_render_configuration_sweep(gpu_lib):
