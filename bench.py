@@ -291,7 +291,7 @@ def bench_frame(args, workload):
             # shared by neighbouring samples are counted once per sample), so it is no fraction of the peak
             roof["traffic"] = None
             roof["achieved"] = conv
-            roof["frac"] = round(conv / HBM_PEAK_GBS, 4) if conv <= HBM_PEAK_GBS else None
+            roof["frac"] = None
             roof["basis"] = "gather-convention bytes / launch duration (no counter run covers this configuration)"
     roof["avg_launch_ms"] = round(avg_ms, 4)
     roof["launches_per_frame"] = launches
@@ -406,7 +406,8 @@ def bench_gather(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"c2_gather_3x{res}^2x64ch_{M}q_{'coherent' if args.coherent else 'random'}"},
         "roofline": {"kernel": "k_density_xyz", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     # sorted queries share texels: their algorithmic rate is cache-served and no fraction of the peak
+                     "unit": "GB/s", "frac": None if args.coherent else round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "avg_launch_ms": round(ker_ms, 4), "bytes_per_query": Bq},
         "cpu_baseline": cpu,
     }
