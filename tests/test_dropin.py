@@ -71,3 +71,31 @@ def test_wrapped_reference_model_renders_the_fixture(gpu_lib, kind, name):
         wrapped.alpha_mask_filter_thre = 2.0  # nothing passes
         none, _ = wrapped(d["rays"], app_code=code, N_samples=cfg["N_samples"])
         assert bool((none["rgb_map"] == 1.0).all()) and bool((none["depth_map"] == 0.0).all())
+
+
+def _psnr(img, gt):
+    return float(-10.0 * torch.log10(torch.mean((img - gt) ** 2)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,name", CASES)
+def test_render_check_in_the_reference_tests_style(gpu_lib, kind, name):
+    """The reference's render tests call renderer_fn on a loaded model and assert that the PSNR against the
+    ground-truth images stays within 5 % of a recorded baseline (`assert base / new - 1 <= 0.05`, tests/utils.py:14-20).
+    Same check here: ground truth = the fixture's image plus seeded noise (about 26 dB, the range of the reference's
+    baselines), baseline = the PSNR of the reference's own output, new = the wrapped model through renderer_fn in
+    the reference's default chunks."""
+    from landmark_amd.model import from_reference_model
+    from landmark_amd.render import renderer_fn
+
+    p, d, cfg = load_golden(name, kind)
+    gt = (d["rgb_map"] + 0.05 * torch.randn(d["rgb_map"].shape, generator=torch.Generator().manual_seed(7))).clamp(0, 1)
+    base = _psnr(d["rgb_map"], gt)
+    gridnerf = from_reference_model(reference_model_stub(p, args_as_dict=(kind == "stacked")), device="cuda")
+    kw = {} if cfg.get("app_code") is None else {"app_code": cfg["app_code"]}
+    ret, _ = renderer_fn(d["rays"], gridnerf, chunk=4096, N_samples=cfg["N_samples"], white_bg=True, is_train=False,
+                         device="cuda", **kw)
+    new = _psnr(ret["rgb_map"].cpu(), gt)
+    assert 20.0 < base < 40.0
+    assert base / new - 1 <= 0.05
+    assert abs(base - new) < 1e-3  # far inside the reference's band: the two images differ by 1e-4 at most
