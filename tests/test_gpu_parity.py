@@ -183,6 +183,39 @@ def test_sample_cull_edge_cases(gpu_lib):
     assert _model(p).sample_cull(rays)["n_valid"] == 0
 
 
+@pytest.mark.parametrize("opt,S,mask", [(1, 128, True), (0, 100, True), (1, 64, False), (0, 200, False)])
+def test_non_finite_rays_do_not_disturb_their_neighbours(gpu_lib, opt, S, mask):
+    """Rays with NaN or infinite components (a degenerate pose, a normalised zero vector) and rays along the axes
+    (zero direction components: the sampler's 1e-6 substitute) sit between ordinary rays of a chunk.  Every
+    address the kernels form stays inside the tables whatever the coordinates, and the ordinary rays come out as
+    they do without the others, bit for bit."""
+    p = _scene(opt=opt, S=S, with_mask=mask, step_ratio=0.3)
+    m = _model(p, mlp_precision="f16x2")
+    good = scenes.pinhole_rays(48, 40, 42.0, scenes.sphere_pose(2.5, 9))
+    nan, inf = float("nan"), float("inf")
+    odd = torch.tensor([
+        [nan, 0.0, 0.0, 0.0, 0.0, -1.0], [0.0, 0.0, 2.0, nan, nan, nan], [nan] * 6,
+        [inf, 0.0, 0.0, 0.0, 0.0, -1.0], [0.0, 0.0, 2.0, inf, 0.0, -1.0], [0.0, 0.0, -inf, 0.0, 0.0, 1.0],
+        [0.0, 0.0, 2.0, 0.0, 0.0, 0.0], [0.1, -0.2, 2.0, 0.0, 0.0, -1.0], [2.0, 0.1, 0.0, -1.0, 0.0, 0.0],
+        [0.0, 0.0, 2.0, 0.0, 0.0, -1e30], [1e30, 1e30, 1e30, -1.0, -1.0, -1.0], [0.0, 0.0, 2.0, 1e-30, 0.0, -1e-30],
+    ])
+    mixed = good.clone()
+    where = torch.arange(odd.shape[0]) * 157 + 3
+    mixed[where] = odd
+    keep = torch.ones(good.shape[0], dtype=torch.bool)
+    keep[where] = False
+    want = m(good, N_samples=S)[0]
+    got = m(mixed, N_samples=S)[0]
+    assert torch.equal(got["rgb_map"].cpu()[keep], want["rgb_map"].cpu()[keep])
+    assert torch.equal(got["depth_map"].cpu()[keep], want["depth_map"].cpu()[keep])
+    # the axis-parallel rays are ordinary input for the reference: against the oracle
+    axis = odd[7:9]
+    ref = O.render_chunk(p, axis, N_samples=S)
+    out = m(axis, N_samples=S)[0]
+    assert (out["rgb_map"].cpu() - ref["rgb_map"]).abs().max().item() <= RGB_TOL_F32
+    assert (out["depth_map"].cpu() - ref["depth_map"]).abs().max().item() <= RGB_TOL_F32
+
+
 # ------------------------------------------------------------------------------------ part 2
 @pytest.mark.parametrize("ndims,res,dn,an", [(3, (1,), 16, 48), (1, (1, 2, 4), 16, 48), (3, (1, 2), 64, 64), (2, (1,), 8, 16)])
 def test_gather_matches_grid_sample(gpu_lib, ndims, res, dn, an):
