@@ -716,6 +716,21 @@ def test_render_frame_from_pose(gpu_lib):
     for n in (1, 3):
         img_n, dep_n = render_frame(m, pose, H, W, chunk=20 * W, depth=True, streams=n)
         assert torch.equal(img_n, img) and torch.equal(dep_n, dep)
+    # a workspace sized far too small, on a frame large enough to pass the floors of the adaptive sizing: the chunks
+    # of both streams overflow, are repeated after the streams join, and the frame comes out as on a worst-case
+    # workspace; the model remembers the room it needed
+    H2, W2 = 144, 192
+    pose2 = torch.cat([scenes.orbit_pose(2.6, 1.9, 3), torch.tensor([[0.0], [0.0], [2 * focal]])], 1)
+    img_w, dep_w = render_frame(_model(p, mlp_precision="f16x2", capacity="worst"), pose2, H2, W2, chunk=72 * W2, depth=True)
+    tight = _model(p, mlp_precision="f16x2")
+    tight.small_workspace = 0
+    tight.samples_per_ray = [0.5, 0.05]
+    img_t, dep_t = render_frame(tight, pose2, H2, W2, chunk=72 * W2, depth=True)
+    assert torch.equal(img_t, img_w) and torch.equal(dep_t, dep_w)
+    assert tight.samples_per_ray[0] > 0.5 and tight.samples_per_ray[1] > 0.05
+    before = list(tight.samples_per_ray)
+    img_t, _ = render_frame(tight, pose2, H2, W2, chunk=72 * W2, depth=True)
+    assert torch.equal(img_t, img_w) and tight.samples_per_ray == before
 
 
 # ------------------------------------------------------------------------------------ occupancy volume from the model
