@@ -420,8 +420,11 @@ class GridNeRFHIP:
         return self
 
     @torch.no_grad()
-    def forward(self, rays_chunk, app_code=None, white_bg=True, is_train=False, N_samples=-1, idxs_chunk=None):
-        """GridBaseSequential.forward in render mode -> ({"rgb_map","depth_map"}, {})."""
+    def forward(self, rays_chunk, app_code=None, white_bg=True, is_train=False, N_samples=-1, idxs_chunk=None,
+                chunk=None, streams=1):
+        """GridBaseSequential.forward in render mode -> ({"rgb_map","depth_map"}, {}).  Two arguments the reference
+        does not have: `chunk` = rays per lm_render call (default: as many as one launch and the workspace budget
+        take) and `streams` = how many streams the chunks of this call are dealt to (see render_chunks)."""
         if is_train:
             raise NotImplementedError("training is outside this render path (is_train must be False)")
         if idxs_chunk is not None:
@@ -433,17 +436,46 @@ class GridNeRFHIP:
         N = rays.shape[0]
         rgb = torch.empty((N, 3), dtype=torch.float32, device=self.device)
         depth = torch.empty((N,), dtype=torch.float32, device=self.device)
-        step = self.preferred_chunk(N, N_samples) if N else 1  # a call of any size: split where one launch cannot take it
-        starts = list(range(0, N, step))
-        counters = torch.zeros((max(len(starts), 1), L.LM_STAT_WORDS), dtype=torch.int32, device=self.device)
-        for ci, start in enumerate(starts):
-            sl = slice(start, min(start + step, N))
-            self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, counters=counters[ci])
-        self.finish_chunks([(slice(st, min(st + step, N)), counters[ci]) for ci, st in enumerate(starts)], rays, rgb, depth,
-                           white_bg=white_bg, N_samples=N_samples)
-        if starts:
-            self.counters.copy_(counters[len(starts) - 1])
+        if N:
+            # a call of any size: split where one launch cannot take it
+            step = self.preferred_chunk(N, N_samples) if chunk is None else max(1, int(chunk))
+            self.render_chunks(rays, rgb, depth, step, white_bg=white_bg, N_samples=N_samples, streams=streams)
         return {"rgb_map": rgb, "depth_map": depth}, {}
+
+    def render_chunks(self, rays, rgb, depth, step, white_bg=True, N_samples=-1, streams=1) -> int:
+        """Render rays[N,6] into rgb[N,3] / depth[N] in chunks of `step` rays, the chunks dealt in turn to `streams`
+        streams: the current one and side streams of the same priority, each with a workspace and a counter block
+        of its own, so that the compute-bound stages of one chunk run under the memory-bound stages of another (and
+        small chunks, which cannot fill the GPU, run side by side).  The current stream continues after all of
+        them; chunks whose workspace overflowed are then repeated (finish_chunks).  Returns the number of chunks."""
+        N = rays.shape[0]
+        S = self._samples_for(N_samples)
+        if step * S >= 2**32:
+            raise L.LandmarkError(f"{step} rays x {S} samples do not fit 32-bit sample indices; use smaller chunks")
+        starts = list(range(0, N, step))
+        if not starts:
+            return 0
+        current = torch.cuda.current_stream(self.device)
+        side = self.side_streams(min(int(streams), len(starts)) - 1) if streams > 1 and len(starts) > 1 else []
+        counters = torch.zeros((len(starts), L.LM_STAT_WORDS), dtype=torch.int32, device=self.device)  # a block per chunk
+        if side:
+            ready = torch.cuda.Event()
+            ready.record(current)
+            for s in side:
+                s.wait_event(ready)
+        lanes = [current] + side
+        done = []
+        for i, start in enumerate(starts):
+            sl = slice(start, min(start + step, N))
+            with torch.cuda.stream(lanes[i % len(lanes)]):
+                self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, slot=i % len(lanes),
+                                 counters=counters[i])
+            done.append((sl, counters[i]))
+        for s in side:
+            current.wait_stream(s)
+        self.finish_chunks(done, rays, rgb, depth, white_bg=white_bg, N_samples=N_samples)
+        self.counters.copy_(counters[len(starts) - 1])
+        return len(starts)
 
     __call__ = forward
 

@@ -27,6 +27,11 @@ def renderer_fn(rays, gridnerf, chunk=4096, N_samples=-1, white_bg=True, is_trai
     chunk = int(chunk)
     if not exact_chunk and idxs is None and n_all > chunk and hasattr(gridnerf, "preferred_chunk"):
         chunk = max(chunk, gridnerf.preferred_chunk(n_all, N_samples))
+    if exact_chunk and idxs is None and not is_train and hasattr(gridnerf, "render_chunks"):
+        # the reference's slicing, but one call: outputs allocated once, the chunks dealt to four streams (a chunk
+        # of a few thousand rays cannot fill the GPU, four of them side by side come closer)
+        return gridnerf(rays.to(device), is_train=False, white_bg=white_bg, N_samples=N_samples, chunk=chunk, streams=4,
+                        **extra_kw)
     for ci in range(n_all // chunk + int(n_all % chunk > 0)):
         rays_chunk = rays[ci * chunk : (ci + 1) * chunk].to(device)
         if idxs is not None:
@@ -140,29 +145,11 @@ def render_frame(gridnerf, single_pose, H, W, focal=None, chunk=1 << 19, app_cod
         chunk = max(8 * W, int(chunk) // (8 * W) * (8 * W))
     rgb = torch.empty((N, 3), dtype=torch.float32, device=gridnerf.device)
     dep = torch.empty((N,), dtype=torch.float32, device=gridnerf.device)
-    starts = list(range(0, N, chunk))
-    current = torch.cuda.current_stream(gridnerf.device)
-    side = gridnerf.side_streams(min(int(streams), len(starts)) - 1) if streams > 1 and len(starts) > 1 else []
     gridnerf._set_app_code(gridnerf.mlp_precision, app_code)
-    counters = torch.zeros((len(starts), 16), dtype=torch.int32, device=gridnerf.device)  # one block per chunk
-    if side:
-        ready = torch.cuda.Event()
-        ready.record(current)
-        for s in side:
-            s.wait_event(ready)
-    lanes = [current] + side
     saved = gridnerf.ray_row_length
     gridnerf.ray_row_length = W if W % 8 == 0 else 0
     try:
-        done = []
-        for i, start in enumerate(starts):
-            sl = slice(start, min(start + chunk, N))
-            with torch.cuda.stream(lanes[i % len(lanes)]):
-                gridnerf.render_into(rays[sl], rgb[sl], dep[sl], white_bg=white_bg, slot=i % len(lanes), counters=counters[i])
-            done.append((sl, counters[i]))
-        for s in side:
-            current.wait_stream(s)
-        gridnerf.finish_chunks(done, rays, rgb, dep, white_bg=white_bg)  # repeats chunks whose workspace overflowed
+        gridnerf.render_chunks(rays, rgb, dep, chunk, white_bg=white_bg, streams=streams)
     finally:
         gridnerf.ray_row_length = saved
     image = postprocess_rgba8(rgb, H, W, host_image)
