@@ -421,10 +421,11 @@ class GridNeRFHIP:
 
     @torch.no_grad()
     def forward(self, rays_chunk, app_code=None, white_bg=True, is_train=False, N_samples=-1, idxs_chunk=None,
-                chunk=None, streams=1):
+                chunk=None, streams=2):
         """GridBaseSequential.forward in render mode -> ({"rgb_map","depth_map"}, {}).  Two arguments the reference
         does not have: `chunk` = rays per lm_render call (default: as many as one launch and the workspace budget
-        take) and `streams` = how many streams the chunks of this call are dealt to (see render_chunks)."""
+        take) and `streams` = how many streams the chunks of this call are dealt to (see render_chunks; a call that is
+        one chunk stays on the current stream)."""
         if is_train:
             raise NotImplementedError("training is outside this render path (is_train must be False)")
         if idxs_chunk is not None:
