@@ -43,6 +43,45 @@ def test_struct_sizes_match_header_layout():
     assert C.sizeof(L.LmModel) % 8 == 0
 
 
+def test_header_compiles_as_c_and_matches_the_binding_field_by_field(tmp_path):
+    """The header is plain C (gcc -std=c11 -pedantic), and every field of its three structs sits at the offset and
+    has the size the ctypes mirror gives it: a C caller and the Python binding see the same memory."""
+    import shutil
+    import subprocess
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    pairs = [("lm_plane", L.LmPlane), ("lm_geom", L.LmGeom), ("lm_model", L.LmModel)]
+    lines = ['#include "landmark_hip.h"', "#include <stddef.h>", "#include <stdio.h>", "int main(void) {"]
+    for cname, st in pairs:
+        lines.append(f'  printf("{cname} . %zu %zu\\n", (size_t)0, sizeof({cname}));')
+        for field, _ in st._fields_:
+            lines.append(f'  printf("{cname} {field} %zu %zu\\n", offsetof({cname}, {field}), sizeof((({cname} *)0)->{field}));')
+    lines += ['  printf("const LM_ABI_VERSION %d 0\\n", LM_ABI_VERSION);', '  printf("const LM_STAT_WORDS %d 0\\n", LM_STAT_WORDS);',
+              '  printf("const LM_STAT_OVERFLOW %d 0\\n", LM_STAT_OVERFLOW);', '  printf("const LM_MAX_PLANES %d 0\\n", LM_MAX_PLANES);',
+              '  printf("const LM_STATIC_WORKSPACE_BYTES %u 0\\n", (unsigned)LM_STATIC_WORKSPACE_BYTES);', "  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines) + "\n")
+    exe = tmp_path / "layout"
+    subprocess.check_call([cc, "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                           str(src), "-o", str(exe)])
+    seen = {}
+    for row in subprocess.check_output([str(exe)], text=True).splitlines():
+        a, b, off, size = row.split()
+        seen[(a, b)] = (int(off), int(size))
+    for cname, st in pairs:
+        assert seen[(cname, ".")][1] == C.sizeof(st), cname
+        for field, _ in st._fields_:
+            d = getattr(st, field)
+            assert seen[(cname, field)] == (d.offset, d.size), (cname, field)
+    assert seen[("const", "LM_ABI_VERSION")][0] == L.LM_ABI_VERSION
+    assert seen[("const", "LM_STAT_WORDS")][0] == L.LM_STAT_WORDS
+    assert seen[("const", "LM_STAT_OVERFLOW")][0] == L.LM_STAT_OVERFLOW
+    assert seen[("const", "LM_MAX_PLANES")][0] == L.LM_MAX_PLANES
+    assert seen[("const", "LM_STATIC_WORKSPACE_BYTES")][0] == L.LM_STATIC_WORKSPACE_BYTES
+
+
 def test_argument_validation_returns_status_not_abort(lib):
     g = L.LmGeom()
     g.S = 0
