@@ -120,10 +120,11 @@ def bench_frame(args, workload):
         name = f"prod_1080p_aabb_sampler_P1_L3_base{args.base}_step{args.step_ratio:g}_encodeapp_nonlinear"
         app_code = 3
     elif workload == "c1":
-        p = scenes.c1_scene(dense=args.density_shift == 0.0, device=dev)
+        # sampling_opt 0: 3.47 grid cells per step make nSamples 128 and the steps span the box diagonal
+        p = scenes.c1_scene(dense=args.density_shift == 0.0, device=dev, sampling_opt=args.sampling_opt, step_ratio=3.47 if args.sampling_opt == 0 else 2.0)
         H, W = 400, 400
         rays = scenes.c1_rays(H, W, device=dev)
-        name = f"c1_tiny_400x400_shift{args.density_shift:g}"
+        name = f"c1_tiny_400x400_shift{args.density_shift:g}_{'hull' if args.sampling_opt else 'aabb_step3.47'}_S128"
     elif workload == "c5":
         p = scenes.c5_scene(res=args.base * 8, device=dev, density_shift=args.density_shift)
         H, W = 2160, 3840
@@ -154,8 +155,8 @@ def bench_frame(args, workload):
     done = []
     for ci in range(n_chunks):
         sl = slice(ci * chunk, min((ci + 1) * chunk, N))
-        model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci])
-        done.append((sl, counters[ci]))
+        caps = model.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=counters[ci])
+        done.append((sl, counters[ci], caps))
     repeats = model.finish_chunks(done, rays, rgb, depth, white_bg=True)
     ws = model.workspace(chunk, S)
     log(f"[bench] workspace {ws.numel() / 1e9:.2f} GB for chunks of {chunk} rays ({repeats} chunk renders repeated while sizing it; "
@@ -296,7 +297,7 @@ def bench_frame(args, workload):
     roof["avg_launch_ms"] = round(avg_ms, 4)
     roof["launches_per_frame"] = launches
 
-    cpu, parity = cpu_baseline_frame(args, p, rays, rgb, depth, H, W, app_code)
+    cpu, parity = cpu_baseline_frame(args, model, p, rays, rgb, depth, H, W, app_code)
     mrays = N / (ms_step * 1e-3) / 1e6
     out = {
         "metric": "render_throughput", "value": round(mrays, 3), "unit": "Mrays/s", "n_gpus": 1,
@@ -317,9 +318,25 @@ def bench_frame(args, workload):
         # the same frame in two more settings, timed in this run after the region above (never `value`):
         # the reference-semantics mode (fp32 matrix products, no early termination) and the one-orientation model
         steps = max(3, args.steps // 2)
+
+        def timed_complete(mod, ck, what):
+            """ms per frame of `mod`, after a sizing frame and with the overflow counters checked after the timed ones."""
+            nck = (N + ck - 1) // ck
+            cn = torch.zeros((nck, L.LM_STAT_WORDS), dtype=torch.int32, device=dev)
+            sized = []
+            for ci in range(nck):
+                sl = slice(ci * ck, min((ci + 1) * ck, N))
+                caps = mod.render_into(rays[sl], rgb[sl], depth[sl], white_bg=True, counters=cn[ci])
+                sized.append((sl, cn[ci], caps))
+            mod.finish_chunks(sized, rays, rgb, depth, white_bg=True)
+            ms = time_frames(mod, rays, rgb, depth, ck, steps, 2, cn)
+            dropped = int((cn[:, L.LM_STAT_OVERFLOW].cpu().long() & 0xFFFFFFFF).sum())
+            if dropped:
+                raise RuntimeError(f"{what}: {dropped} rays did not fit the workspace capacity: the timed frames are incomplete")
+            return round(ms, 4)
+
         model.mlp_precision, model.term_eps = "f32", 0.0
-        out["ms_per_step_exact"] = {"mlp": "f32", "term_eps": 0.0,
-                                    "ms": round(time_frames(model, rays, rgb, depth, chunk, steps, 2), 4)}
+        out["ms_per_step_exact"] = {"mlp": "f32", "term_eps": 0.0, "ms": timed_complete(model, chunk, "exact mode")}
         del model
         torch.cuda.empty_cache()
         if args.planes != 1:
@@ -327,14 +344,17 @@ def bench_frame(args, workload):
             m1 = GridNeRFHIP(p1, device=dev, mlp_precision=args.mlp, term_eps=term_eps, release_source=True)
             c1 = frame_chunks(m1, N, S, W, args.chunk, not args.no_row_hint)
             out["ms_per_step_P1"] = {"workload": f"c4_1080p_multires_P1_base{args.base}_shift{args.density_shift:g}",
-                                     "ms": round(time_frames(m1, rays, rgb, depth, c1, steps, 2), 4)}
+                                     "ms": timed_complete(m1, c1, "one-orientation model")}
     return out
 
 
-def cpu_baseline_frame(args, p, rays, rgb, depth, H, W, app_code=None):
-    """The CPU oracle on a bounded sample of the frame (evenly spaced scan-lines)."""
+def cpu_baseline_frame(args, model, p, rays, rgb, depth, H, W, app_code=None):
+    """The CPU oracle on a bounded sample of the frame (evenly spaced scan-lines), timed as the CPU baseline, and the
+    parity of the frame just rendered against it: sample-mask mismatches, valid-index and depth-table equality,
+    sample counts of the library's own counters, and the two maxima."""
     if args.no_cpu:
         return None, None
+    from landmark_amd import _lib as L
     from oracle import gridnerf_oracle as O
 
     S = p.n_importance if p.sampling_opt else p.nSamples
@@ -344,68 +364,107 @@ def cpu_baseline_frame(args, p, rays, rgb, depth, H, W, app_code=None):
     t0 = time.time()
     pc = p.to("cpu")
     log(f"[bench] cpu copy of the model {time.time() - t0:.1f}s")
-    r = rays[idx.to(rays.device)].cpu()
+    r_dev = rays[idx.to(rays.device)].contiguous()
+    r = r_dev.cpu()
     torch.set_num_threads(os.cpu_count() if args.cpu_threads <= 0 else args.cpu_threads)
-    t0 = time.perf_counter()
-    ret, _ = O.renderer_fn(r, pc, chunk=8192, white_bg=True, **({} if app_code is None else {"app_code": app_code}))
-    dt = time.perf_counter() - t0
-    d_rgb = (rgb[idx.to(rgb.device)].cpu() - ret["rgb_map"]).abs().max().item()
-    d_dep = (depth[idx.to(rgb.device)].cpu() - ret["depth_map"]).abs().max().item()
+    kw = {} if app_code is None else {"app_code": app_code}
+    ref = {k: [] for k in ("rgb_map", "depth_map", "ray_valid", "z_vals", "band")}
+    n_app_ref, dt = 0, 0.0
+    for i in range(0, r.shape[0], 8192):  # the reference's chunk loop (app/tools/render_utils.py:15-63), chunk 8192
+        t0 = time.perf_counter()
+        ret = O.render_chunk(pc, r[i:i + 8192], white_bg=True, return_aux=True, **kw)
+        dt += time.perf_counter() - t0  # only the render counts as the baseline, not the bookkeeping below
+        ret["band"] = ((ret["weight"] - p.rayMarch_weight_thres).abs() < 2e-7).any(-1)
+        n_app_ref += int(ret["app_mask"].sum())
+        for k in ref:
+            ref[k].append(ret[k])
+    ref = {k: torch.cat(v) for k, v in ref.items()}
     cpu = {"value": round(r.shape[0] / dt / 1e6, 5), "unit": "Mrays/s", "cores": torch.get_num_threads(), "kind": "port",
            "sample": f"{len(ys)} evenly spaced scan-lines ({r.shape[0]} rays) of the same frame, PyTorch oracle, "
                      f"chunk 8192, {dt:.1f}s"}
-    parity = {"rays_checked": int(r.shape[0]), "max_abs_rgb": d_rgb, "max_abs_depth": d_dep}
+    # ---- parity of this run's frame (untimed): decisions bit for bit, rgb / depth maxima
+    got_rgb, got_dep = rgb[idx.to(rgb.device)].cpu(), depth[idx.to(rgb.device)].cpu()
+    d_rgb = (got_rgb - ref["rgb_map"]).abs().max(-1).values
+    d_dep = (got_dep - ref["depth_map"]).abs()
+    cull = model.sample_cull(r_dev)
+    mism = int((cull["ray_valid"].cpu() != ref["ray_valid"]).sum())
+    idx_equal = torch.equal(cull["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
+    z_mism = int((cull["z_vals"].cpu() != ref["z_vals"]).sum())
+    del cull
+    # the whole-chunk render of the same rays on their own: its counters against the oracle's counts, and its
+    # pixels against the frame's (rays are independent: the same bits whatever chunk a ray arrives in)
+    sub, _ = model(r_dev, white_bg=True, **kw)
+    cnt = model.last_counts()
+    ok = ~ref["band"]
+    parity = {
+        "rays_checked": int(r.shape[0]), "samples_checked": int(ref["ray_valid"].numel()),
+        "mask_mismatches": mism, "valid_idx_equal": bool(idx_equal), "z_mismatches": z_mism,
+        "valid_samples": {"oracle": int(ref["ray_valid"].sum()), "lm_render_counter": cnt["n_valid"]},
+        "app_samples": {"oracle": n_app_ref, "lm_render_counter": cnt["n_app"]},
+        "app_mask_band_rays": int(ref["band"].sum()),
+        "max_abs_rgb": d_rgb.max().item(), "max_abs_depth": d_dep.max().item(),
+        "max_abs_rgb_outside_band": d_rgb[ok].max().item(), "max_abs_depth_outside_band": d_dep[ok].max().item(),
+        "chunk_invariant": bool(torch.equal(sub["rgb_map"].cpu(), got_rgb) and torch.equal(sub["depth_map"].cpu(), got_dep)),
+        "note": "mask = AABB and occupancy decisions of every sample of the checked rays (lm_sample_cull vs oracle); band = rays "
+                "holding a weight within 2e-7 of the appearance threshold, whose appearance mask may legitimately differ",
+    }
     return cpu, parity
 
 
 # ----------------------------------------------------------------------------------------
 def bench_gather(args):
-    """Second benchmark configuration: isolated plane/line gather, 3 planes 2048^2 x 64 ch fp32, 2^24 queries."""
+    """Second benchmark configuration: isolated plane/line gather, 3 planes 2048^2 x 64 ch fp32, 2^24 queries.
+    Density form (default): sum over planes and channels -> [M].  Appearance form (--app-mode): the products
+    themselves -> [M, 3*64]."""
     from landmark_amd import scenes
     from landmark_amd.model import GridNeRFHIP
 
     dev = "cuda:0"
     res = args.base * 2
-    p = scenes.make_params(seed=2, gridSize=(res, res, res), ndims=3, resMode=(1,), density_n_comp=64, app_n_comp=16,
-                           device=dev, feature_init="uniform")
-    model = GridNeRFHIP(p, device=dev)
+    app = bool(args.app_mode)
+    p = scenes.make_params(seed=2, gridSize=(res, res, res), ndims=3, resMode=(1,), density_n_comp=4 if app else 64,
+                           app_n_comp=64 if app else 16, device=dev, feature_init="uniform")
+    model = GridNeRFHIP(p, device=dev, release_source=True)
     M = args.queries
     g = torch.Generator(device=dev).manual_seed(2)
     xyz = torch.rand((M, 3), device=dev, generator=g) * 2 - 1
     if args.coherent:
         xyz = xyz[torch.argsort((xyz[:, 0] * 64).floor() * 4096 + (xyz[:, 1] * 64).floor())]
-    out = model.compute_densityfeature(xyz)
+    run = model.app_products if app else model.compute_densityfeature
+    out = run(xyz)
     for _ in range(args.warmup):
-        model.compute_densityfeature(xyz)
+        out = run(xyz)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     ev[0].record()
     for k in range(args.steps):
-        out = model.compute_densityfeature(xyz)
+        out = run(xyz)
         ev[k + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ker_ms = sum(ev[k].elapsed_time(ev[k + 1]) for k in range(args.steps)) / args.steps
-    Bq = plane_bytes_per_sample(model._density) + 12 + 4
+    planes = model._app if app else model._density
+    Bq = plane_bytes_per_sample(planes) + 12 + (4 * model.K_app if app else 4)
     gbs = M * Bq / (ker_ms * 1e-3) / 1e9
     cpu = None
     if not args.no_cpu:
         from oracle import gridnerf_oracle as O
 
-        pc, sub = p.to("cpu"), xyz[: 1 << 20].cpu()
+        n = 1 << (18 if app else 20)
+        pc, sub = p.to("cpu"), xyz[:n].cpu()
         t0 = time.perf_counter()
-        ref = O.density_feature(pc, sub)
+        ref = O.app_products(pc, sub) if app else O.density_feature(pc, sub)
         cdt = time.perf_counter() - t0
-        err = (out[: 1 << 20].cpu() - ref).abs().max().item()
+        err = (out[:n].cpu() - ref).abs().max().item()
         cpu = {"value": round(sub.shape[0] / cdt / 1e6, 4), "unit": "Mqueries/s", "cores": torch.get_num_threads(),
-               "kind": "port", "sample": f"first 2^20 queries, F.grid_sample oracle, {cdt:.1f}s, max|diff| {err:.2e}"}
+               "kind": "port", "sample": f"first {n} queries, F.grid_sample oracle, {cdt:.1f}s, max|diff| {err:.2e}"}
     return {
         "metric": "gather_throughput", "value": round(M / (dt / args.steps) / 1e6, 2), "unit": "Mqueries/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt / args.steps * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"c2_gather_3x{res}^2x64ch_{M}q_{'coherent' if args.coherent else 'random'}"},
-        "roofline": {"kernel": "k_density_xyz", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+        "config": {"workload": f"c2_gather_3x{res}^2x64ch_{M}q_{'coherent' if args.coherent else 'random'}_{'app' if app else 'density'}"},
+        "roofline": {"kernel": "k_app_xyz" if app else "k_density_xyz", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      # sorted queries share texels: their algorithmic rate is cache-served and no fraction of the peak
                      "unit": "GB/s", "frac": None if args.coherent else round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                      "avg_launch_ms": round(ker_ms, 4), "bytes_per_query": Bq},
@@ -496,7 +555,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--host-io", action="store_true", help="also time the frame with rays and results in pinned host memory")
     ap.add_argument("--no-row-hint", action="store_true", help="do not tell the library that rays are image rows")
-    ap.add_argument("--calib", action="store_true", help="also run one 1 GiB device copy (counter calibration)")
+    ap.add_argument("--calib", action="store_true", help="accepted and ignored: the copy and streaming yardsticks run every time")
+    ap.add_argument("--app-mode", action="store_true", help="c2: the appearance form of the gather ([M, 3*64] products out)")
+    ap.add_argument("--sampling-opt", type=int, default=1, choices=[0, 1],
+                    help="c1: 1 = hull sampler (n_importance 128), 0 = equal-step sampler, 128 steps of 3.47 grid cells")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build renders on one GPU; rays are independent, so more GPUs would each take a slice of "
@@ -506,40 +568,33 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
-    copy_rate = stream_rate = None
-    if args.calib:
-        a = torch.ones(1 << 28, device="cuda:0")  # 1 GiB read + 1 GiB written by one copy kernel
-        b = torch.empty_like(a)
-        b.copy_(a)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(20):
-            b.copy_(a)
-        e1.record()
-        torch.cuda.synchronize()
-        copy_rate = 20 * 2 * a.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
-        log(f"[bench] device copy, 1 GiB: {copy_rate:.0f} GB/s (read + write)")
-        # a plain streaming kernel (one read, one write per element) as a second yardstick
-        torch.add(a, 1.0, out=b)
+    # yardsticks of this box's memory system, measured in every run (a fraction of a second): a plain 1 GiB device
+    # copy and an elementwise add (1 GiB in, 1 GiB out), bytes read + written per second
+    a = torch.ones(1 << 28, device="cuda:0")
+    b = torch.empty_like(a)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    rates = []
+    for op in (lambda: b.copy_(a), lambda: torch.add(a, 1.0, out=b)):
+        op()
         torch.cuda.synchronize()
         e0.record()
         for _ in range(20):
-            torch.add(a, 1.0, out=b)
+            op()
         e1.record()
         torch.cuda.synchronize()
-        stream_rate = 20 * 2 * a.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9
-        log(f"[bench] elementwise add, 1 GiB in, 1 GiB out: {stream_rate:.0f} GB/s (read + write)")
-        del a, b
+        rates.append(20 * 2 * a.numel() * 4 / (e0.elapsed_time(e1) * 1e-3) / 1e9)
+    copy_rate, stream_rate = rates
+    log(f"[bench] 1 GiB device copy {copy_rate:.0f} GB/s, elementwise add {stream_rate:.0f} GB/s (read + write)")
+    del a, b
+    torch.cuda.empty_cache()
     if args.workload == "c2":
         out = bench_gather(args)
     elif args.workload == "c3":
         out = bench_mlp(args)
     else:
         out = bench_frame(args, args.workload)
-    if copy_rate is not None:
-        out["hbm_copy_GBps"] = round(copy_rate, 1)
-        out["hbm_stream_GBps"] = round(stream_rate, 1)
+    out["hbm_copy_GBps"] = round(copy_rate, 1)
+    out["hbm_stream_GBps"] = round(stream_rate, 1)
     print(json.dumps(out), flush=True)
 
 

@@ -7,7 +7,13 @@
  *     parameter is documented as host memory; device pointers must be 16-byte aligned,
  *     except ray arrays ([N,6] floats, any row of a 16-byte aligned array: 8-byte aligned);
  *   - the caller owns every buffer (inputs, outputs and the workspace); the library
- *     allocates nothing and keeps no global state besides a thread-local error string;
+ *     allocates no memory.  State it keeps between calls: per calling thread, the error
+ *     string and a few per-device caches of device facts and kernel attributes (number of
+ *     compute units, resident-workgroup counts, whether a kernel's LDS limit has been
+ *     raised), filled on first use and never invalidated; per process, for
+ *     lm_render_static only, one built-in device array per GPU and a mutex-guarded table of
+ *     those arrays' device addresses.  Nothing of it depends on a model or a call's
+ *     arguments, so calls from different threads never interact unless they share buffers;
  *   - every function takes the HIP stream to launch on (`void*` = hipStream_t, NULL =
  *     the null stream) and returns without waiting for the GPU;
  *   - return value: LM_OK (0) or a negative lm_status; lm_last_error() describes the
@@ -144,9 +150,12 @@ typedef struct lm_model {
     /* Workspace capacities of one lm_render call, in samples: room for the chunk's valid samples and for its
      * appearance samples (weight > weight_thres).  0 = the worst case (every sample valid, every ray with
      * min(S, 1 / weight_thres) appearance samples), which cannot overflow; the reference's fused path sizes its
-     * buffers for 64 rows per ray instead (dist_render/kernel/cuda_render_extend.py:35-159).  A ray whose samples
-     * do not fit is rendered as if it had none and counted in counters[LM_STAT_OVERFLOW]: the caller reads the
-     * counters, and when that word is not zero repeats the call with capacities of at least
+     * buffers for 64 rows per ray instead (dist_render/kernel/cuda_render_extend.py:35-159).  A ray that does
+     * not fit is counted in counters[LM_STAT_OVERFLOW] and its output is incomplete: a ray whose valid samples
+     * exceed cap_valid is rendered as if it had none (background colour, depth 0); a ray whose appearance samples
+     * exceed cap_app keeps the depth and the accumulated opacity of its march but gets no colour from them (rgb =
+     * 1 - acc on a white background, 0 otherwise).  Either way the pixel is wrong until the call is repeated: the
+     * caller reads the counters, and when OVERFLOW is not zero repeats the call with capacities of at least
      * counters[LM_STAT_N_VALID] and counters[LM_STAT_N_APP] (both keep counting past the capacity; after a
      * valid-sample overflow N_APP is a lower bound and the repeat may report a second, appearance overflow). */
     int64_t cap_valid;

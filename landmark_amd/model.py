@@ -47,6 +47,7 @@ class GridNeRFHIP:
         release_source: bool = False,
         occupancy: str = "auto",  # auto | cells | u8 | f32: storage of the occupancy volume
         capacity: str = "adaptive",  # adaptive | worst: how the render workspace is sized (see `capacities`)
+        check_fp16_range: bool = True,  # refuse f16 / f16x2 for tables whose products can leave the fp16 range
     ):
         if not torch.cuda.is_available():
             raise L.LandmarkError("GridNeRFHIP needs a GPU; there is no CPU path")
@@ -120,12 +121,15 @@ class GridNeRFHIP:
             self._w1_plain = torch.cat([w1[:, :27], w1[:, 27 + self._latent_dim :]], 1).contiguous()  # [128, 150]
         self._packed = {}
         self._bias_code = {}
+        self.check_fp16_range = bool(check_fp16_range)
+        self._fp16_bounds = None
         self._pack_mlp(mlp_precision)
         # --- workspace cache (per-S geometry is cached in _geom_cache)
         self._ws = {}  # workspace per slot (one slot per stream that renders concurrently)
         self._side_streams = []
         self._slot_counters = []
-        self.counters = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)
+        with torch.inference_mode(False):
+            self.counters = torch.zeros(L.LM_STAT_WORDS, dtype=torch.int32, device=self.device)  # copied into per call
 
     @property
     def alpha_mask_filter_thre(self) -> float:
@@ -209,9 +213,44 @@ class GridNeRFHIP:
             out.append(s)
         return out
 
+    FP16_MAX = 65504.0
+
+    def fp16_range_bounds(self) -> Dict[str, float]:
+        """Upper bounds of the magnitudes the fp16 matrix modes (f16, f16x2) carry as fp16 numbers: the plane x line
+        products of the appearance tables (max |plane_k| * max |line_k| over the planes) and the 27 features behind
+        basis_mat (row sums of |basis_mat| weighted with the per-plane product bounds).  One pass over the tables,
+        cached."""
+        if self._fp16_bounds is None:
+            per_plane = []
+            for k in range(len(self._app)):
+                P, Ln = self._tables[2 * (len(self._density) + k)], self._tables[2 * (len(self._density) + k) + 1]
+                (p_lo, p_hi), (l_lo, l_hi) = torch.aminmax(P), torch.aminmax(Ln)  # no temporary of the table's size
+                per_plane.append(max(-float(p_lo), float(p_hi)) * max(-float(l_lo), float(l_hi)))
+            basis = self.p.basis_mat.detach().float().abs().cpu()
+            col = torch.cat([torch.full((pl.C,), b) for pl, b in zip(self._app, per_plane)])
+            self._fp16_bounds = {"product": max(per_plane), "feature": float((basis * col[None]).sum(1).max())}
+        return self._fp16_bounds
+
+    def _check_fp16_range(self, precision: str) -> None:
+        """The fp16 matrix modes turn a product beyond 65504 into inf without any status.  Refuse them for tables whose
+        plane x line products can get there; warn when only the (looser) bound of the projected features does."""
+        if precision not in ("f16", "fp16", "f16x2") or not self.check_fp16_range:
+            return
+        b = self.fp16_range_bounds()
+        if not b["product"] < self.FP16_MAX:
+            raise L.LandmarkError(
+                f"mlp_precision={precision!r}: plane x line products of the appearance tables can reach {b['product']:.3g}, "
+                f"beyond the fp16 range (65504); use mlp_precision='bf16' or 'f32' (or check_fp16_range=False to override)")
+        if not b["feature"] < self.FP16_MAX:
+            import warnings
+
+            warnings.warn(f"mlp_precision={precision!r}: the bound of the projected appearance features is {b['feature']:.3g}, "
+                          "beyond the fp16 range (65504); results turn inf if a feature really gets there", RuntimeWarning)
+
     def _pack_mlp(self, precision: str):
         if precision in self._packed:
             return self._packed[precision]
+        self._check_fp16_range(precision)
         prec = L.MLP_PREC[precision]
         p = self.p
         K = self.K_app
@@ -238,7 +277,10 @@ class GridNeRFHIP:
             ),
             "lm_mlp_pack",
         )
-        dev = torch.from_numpy(host).to(self.device)
+        with torch.inference_mode(False):
+            # updated in place per app_code later on: must not become an inference tensor when the first call
+            # comes from inside torch.inference_mode() (as the serving engine's does)
+            dev = torch.from_numpy(host).to(self.device)
         self._packed[precision] = (prec, dev)
         return self._packed[precision]
 
@@ -386,15 +428,16 @@ class GridNeRFHIP:
     # chunks whose worst-case workspace stays below this are always given the worst case
     small_workspace = 256 << 20
 
-    def preferred_chunk(self, n_rays: int, N_samples: int = -1) -> int:
+    def preferred_chunk(self, n_rays: int, N_samples: int = -1, lanes: int = 1) -> int:
         """Rays per lm_render call when the caller leaves the choice to the library: up to 2^20
         (large launches are what keeps the GPU busy: a 1080p frame in 4096-ray chunks takes 14
-        times as long as in two chunks), as many as `workspace_budget` and 32-bit sample indices allow."""
+        times as long as in two chunks), as many as `workspace_budget` and 32-bit sample indices allow.
+        `lanes`: streams the chunks will be dealt to; each owns a workspace, so the budget is shared among them."""
         S = self._samples_for(N_samples)
         probe = 1 << 16
         m = self._model_struct(S, True, self.capacities(probe, S))
         per_ray = self.lib.lm_render_workspace_bytes(C.byref(m), probe) / probe
-        fit = int(self.workspace_budget / max(per_ray, 1.0))
+        fit = int(self.workspace_budget / max(int(lanes), 1) / max(per_ray, 1.0))
         cap = min(1 << 20, ((1 << 32) - 1) // S, max(fit, 4096))
         return max(1, min(int(n_rays), cap))
 
@@ -439,7 +482,7 @@ class GridNeRFHIP:
         depth = torch.empty((N,), dtype=torch.float32, device=self.device)
         if N:
             # a call of any size: split where one launch cannot take it
-            step = self.preferred_chunk(N, N_samples) if chunk is None else max(1, int(chunk))
+            step = self.preferred_chunk(N, N_samples, lanes=streams) if chunk is None else max(1, int(chunk))
             self.render_chunks(rays, rgb, depth, step, white_bg=white_bg, N_samples=N_samples, streams=streams)
         return {"rgb_map": rgb, "depth_map": depth}, {}
 
@@ -469,9 +512,9 @@ class GridNeRFHIP:
         for i, start in enumerate(starts):
             sl = slice(start, min(start + step, N))
             with torch.cuda.stream(lanes[i % len(lanes)]):
-                self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, slot=i % len(lanes),
-                                 counters=counters[i])
-            done.append((sl, counters[i]))
+                caps = self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples,
+                                        slot=i % len(lanes), counters=counters[i])
+            done.append((sl, counters[i], caps))
         for s in side:
             current.wait_stream(s)
         self.finish_chunks(done, rays, rgb, depth, white_bg=white_bg, N_samples=N_samples)
@@ -484,30 +527,32 @@ class GridNeRFHIP:
         """Chunks rendered with a workspace below the worst case may have dropped rays: read their counter blocks
         (one small copy, the call's one host synchronisation), raise the capacity to what the counters ask for and
         render the affected chunks again until none overflows.  `chunks`: (slice of the ray array, the counter
-        block its render wrote).  Returns the number of repeated renders; nothing to do with capacity="worst"."""
-        S = self._samples_for(N_samples)
-        # chunks rendered on a worst-case workspace cannot have overflowed: no need to look (or to synchronise)
-        pending = [(sl, c) for sl, c in chunks if self.capacities(sl.stop - sl.start, S) != (0, 0)]
+        block its render wrote, the capacities render_into returned for it).  Returns the number of repeated
+        renders; nothing to do with capacity="worst"."""
+        # chunks rendered on a worst-case workspace cannot have overflowed: no need to look (or to synchronise).
+        # The capacities are the ones each render was launched with: an earlier chunk of the same call may have
+        # raised samples_per_ray since.
+        pending = [(sl, c, caps) for sl, c, caps in chunks if caps != (0, 0)]
         if not pending:
             return 0
         repeats = 0
         for _ in range(6):
-            host = torch.stack([c for _, c in pending]).cpu().long() & 0xFFFFFFFF
+            host = torch.stack([c for _, c, _ in pending]).cpu().long() & 0xFFFFFFFF
             again = []
-            for (sl, cnt), row in zip(pending, host):
+            for (sl, cnt, caps), row in zip(pending, host):
                 if int(row[L.LM_STAT_OVERFLOW]) == 0:
                     continue
                 n = sl.stop - sl.start
-                caps = self.capacities(n, S)
                 valid_over = caps[0] != 0 and int(row[L.LM_STAT_N_VALID]) > caps[0]
                 self._grow_capacity(n, int(row[L.LM_STAT_N_VALID]), int(row[L.LM_STAT_N_APP]), valid_over)
                 again.append((sl, cnt))
             if not again:
                 return repeats
+            pending = []
             for sl, cnt in again:
-                self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, counters=cnt)
+                caps = self.render_into(rays[sl], rgb[sl], depth[sl], white_bg=white_bg, N_samples=N_samples, counters=cnt)
+                pending.append((sl, cnt, caps))
                 repeats += 1
-            pending = again
         raise L.LandmarkError("workspace capacity still overflows after six repeats")
 
     def render_into(self, rays, rgb, depth, white_bg=True, N_samples=-1, counters=None, events=None, slot=0):
@@ -516,10 +561,11 @@ class GridNeRFHIP:
         (enable_timing=True) re-recorded around the stages on the current stream.  Calls that may
         run at the same time (different streams) must use different slots: a slot owns a workspace
         and a counter block.  The workspace has the room `capacities` gives it: unless that is the worst
-        case, counters[LM_STAT_OVERFLOW] tells whether rays were dropped (see finish_chunks)."""
+        case, counters[LM_STAT_OVERFLOW] tells whether rays were dropped (see finish_chunks).  Returns the capacities
+        (valid samples, appearance samples; (0, 0) = worst case) the render was launched with."""
         N = rays.shape[0]
         if N == 0:
-            return
+            return (0, 0)
         S = self._samples_for(N_samples)
         caps = self.capacities(N, S)
         ws = self.workspace(N, S, slot, caps)
@@ -536,6 +582,7 @@ class GridNeRFHIP:
             ),
             "lm_render",
         )
+        return caps
 
     # ------------------------------------------------------------------ occupancy volume from the model
     @torch.no_grad()
@@ -585,6 +632,26 @@ class GridNeRFHIP:
         total = gs[0] * gs[1] * gs[2]
         self.alpha_rest_percent = int(count.item()) / total * 100
         return torch.stack((lo, hi)).to(self.device)
+
+    def save(self, path) -> None:
+        """Write the model in the reference's checkpoint format (GridBaseSequential.save,
+        gridnerf_sequential.py:209-223): kwargs, state dict and the occupancy volume the model holds NOW, i.e. the
+        one updateAlphaMask built if it was called, packed to bits with its box.  Needs the source tensors
+        (not available after release_source=True)."""
+        import copy
+
+        from .checkpoint import save_checkpoint
+
+        if not self.p.density_plane:
+            raise L.LandmarkError("save: the source tables were released (release_source=True)")
+        q = copy.copy(self.p)
+        if self.alphaMask is None:
+            q.alpha_volume, q.alpha_aabb = None, None
+        else:
+            q.alpha_volume = self.alphaMask.alpha_volume.reshape(self.alphaMask.alpha_volume.shape[-3:]).cpu()
+            q.alpha_aabb = self.alphaMask.aabb.detach().float().cpu()
+        q.alpha_mask_filter_thre = self._alpha_mask_filter_thre
+        save_checkpoint(q, path)
 
     def last_counts(self) -> Dict[str, int]:
         """Valid / appearance sample counts of the last chunk (synchronises)."""

@@ -218,10 +218,14 @@ def pinhole_rays(H: int, W: int, focal: float, c2w: torch.Tensor, device="cpu") 
 # --------------------------------------------------------------------------------------
 # the five benchmark configurations
 # --------------------------------------------------------------------------------------
-def c1_scene(dense: bool = False, sampling_opt: int = 1, device="cpu", grid=256) -> GridNeRFParams:
+def c1_scene(dense: bool = False, sampling_opt: int = 1, device="cpu", grid=256, step_ratio: float = 2.0) -> GridNeRFParams:
     """Tiny full render: 3 planes 256^2 + 3 lines 256, 16/48 ch fp32, seed 0.
     `dense=True` uses density_shift 0 so that the colour network actually runs
-    (with the stated init and shift -10 every weight is far below 1e-3)."""
+    (with the stated init and shift -10 every weight is far below 1e-3).
+    `sampling_opt=1`: 128 samples between near and the box floor (hull sampler); `sampling_opt=0`: equal steps of
+    `step_ratio` grid cells from the slab entry (gridnerf_sequential.py:158-164, 260-281): with 128 steps the
+    reference's default ratio 0.5 covers half a scene unit behind the entry point, 3.47 the whole diagonal of the
+    box (and makes nSamples 128)."""
     return make_params(
         seed=0,
         gridSize=(grid, grid, grid),
@@ -232,7 +236,7 @@ def c1_scene(dense: bool = False, sampling_opt: int = 1, device="cpu", grid=256)
         density_shift=0.0 if dense else -10.0,
         sampling_opt=sampling_opt,
         n_importance=128,
-        step_ratio=2.0,
+        step_ratio=step_ratio,
     )
 
 

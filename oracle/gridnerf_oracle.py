@@ -13,6 +13,8 @@ reproducible bit for bit.
 How each function is pinned (tests/test_oracle_*.py):
   sample_ray_aabb / sample_ray_within_hull   closed forms + brute force
   sample_alpha                               scalar trilinear loop, volume invariants
+  sample_and_cull                            the reference's own sub-results in the golden vectors (inside-box mask
+                                             and occupancy lookups of every sample); used by render_chunk
   normalize_coord                            AABB corners -> +-1
   density_feature / app_feature              scalar bilinear loop, affine planes,
                                              texel-centre queries, one-hot column order
@@ -280,25 +282,36 @@ def mlp_render(p, viewdirs, feats, latent=None):
 # whole chunk
 # --------------------------------------------------------------------------------------
 @torch.no_grad()
-def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False, app_code=None):
-    """GridBaseSequential.forward with is_train=False,
-    app/models/gridnerf_sequential.py:448-504 (sampling_opt=0) and :523-576
-    (sampling_opt=1); the two branches differ only in the sampler."""
+def sample_and_cull(p, rays_chunk, N_samples=-1):
+    """The head of GridBaseSequential.forward: the sampler, then the occupancy lookup on the
+    un-normalised points of the samples inside the box, ANDed into the mask with the reference's
+    update idiom (gridnerf_sequential.py:451-465 for sampling_opt=0, :528-541 for sampling_opt=1).
+    Returns (xyz [N,S,3] un-normalised, z [N,S], ray_valid [N,S] bool).  Needs the occupancy volume
+    and the box only, no feature table."""
     rays_o = rays_chunk[:, :3]
-    rays_d = viewdirs = rays_chunk[:, 3:6]
+    viewdirs = rays_chunk[:, 3:6]
     if p.sampling_opt:
         xyz, z, ray_valid = sample_ray_within_hull(p, rays_o, viewdirs, p.n_importance)
     else:
         xyz, z, ray_valid = sample_ray_aabb(p, rays_o, viewdirs, N_samples)
-    dists = torch.cat((z[:, 1:] - z[:, :-1], torch.zeros_like(z[:, :1])), dim=-1)
-    viewdirs = viewdirs.view(-1, 1, 3).expand(xyz.shape)
-
     if p.alpha_volume is not None:
         alphas = sample_alpha(p.alpha_volume, p.alpha_aabb, xyz[ray_valid])
         keep = alphas > p.alpha_mask_filter_thre
         ray_invalid = ~ray_valid
         ray_invalid[ray_valid] |= ~keep
         ray_valid = ~ray_invalid
+    return xyz, z, ray_valid
+
+
+@torch.no_grad()
+def render_chunk(p, rays_chunk, white_bg=True, N_samples=-1, return_aux=False, app_code=None):
+    """GridBaseSequential.forward with is_train=False,
+    app/models/gridnerf_sequential.py:448-504 (sampling_opt=0) and :523-576
+    (sampling_opt=1); the two branches differ only in the sampler."""
+    viewdirs = rays_chunk[:, 3:6]
+    xyz, z, ray_valid = sample_and_cull(p, rays_chunk, N_samples)
+    dists = torch.cat((z[:, 1:] - z[:, :-1], torch.zeros_like(z[:, :1])), dim=-1)
+    viewdirs = viewdirs.view(-1, 1, 3).expand(xyz.shape)
 
     sigma = torch.zeros(xyz.shape[:-1], device=xyz.device)
     rgb = torch.zeros((*xyz.shape[:2], 3), device=xyz.device)

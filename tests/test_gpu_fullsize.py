@@ -137,13 +137,61 @@ def test_full_frame_chunk_invariance_and_background(gpu_lib, frame):
     assert bool(empty.any()) and bool((a["rgb_map"][empty] == 1.0).all()) and bool((black["rgb_map"][empty] == 0.0).all())
 
 
-def test_full_frame_oracle_spot_check(gpu_lib, frame):
+def _frame_sample(rays, H=1080, W=1920):
+    """Rays of the 1080p frame for the oracle: 4096 around the image centre, and a strided sample of the whole
+    frame (every `stride`-th pixel, a stride coprime to the row length so that all columns are visited)."""
+    centre = torch.arange(W * (H // 2) + W // 2 - 4096, W * (H // 2) + W // 2)
+    return centre, torch.arange(0, H * W, 37), torch.arange(0, H * W, 521)
+
+
+def test_full_frame_sample_masks_bit_exact(gpu_lib, frame):
+    """The decisions the benchmark frame is culled with, on the frame's own 256^3 occupancy volume and 1080p
+    camera: valid mask, ascending valid-sample indices and sample depths equal the oracle's bit for bit on 60 000
+    rays spread over the whole frame, and the whole-chunk render counts exactly the oracle's valid samples."""
+    import copy
+
     p, rays, m = frame
-    out, _ = m(rays[: 1920 * 540 + 960][-4096:])  # 4096 rays around the image centre
-    sub = rays[: 1920 * 540 + 960][-4096:].cpu()
-    ref = O.render_chunk(p.to("cpu"), sub, return_aux=True)
+    centre, dense, _ = _frame_sample(rays)
+    idx = torch.unique(torch.cat([centre, dense]))
+    sub = rays[idx.cuda()].contiguous()
+    q = copy.copy(p)  # the mask needs the box, the sampler settings and the occupancy volume only
+    q.aabb, q.alpha_volume, q.alpha_aabb = p.aabb.cpu(), p.alpha_volume.cpu(), p.alpha_aabb.cpu()
+    _, z, valid = O.sample_and_cull(q, sub.cpu())
+    frac = valid.float().mean().item()
+    assert 0.02 < frac < 0.5 and bool(valid.any(-1).any()) and not bool(valid.any(-1).all())
+    cull = m.sample_cull(sub)
+    assert torch.equal(cull["ray_valid"].cpu(), valid)
+    assert torch.equal(cull["valid_idx"].cpu(), valid.reshape(-1).nonzero()[:, 0])
+    assert torch.equal(cull["z_vals"].cpu(), z)
+    assert cull["n_valid"] == int(valid.sum())
+    # lm_render's own cull (a lane per ray and bitmap word, no index list) on the same rays
+    rgb = torch.empty((sub.shape[0], 3), device="cuda")
+    dep = torch.empty((sub.shape[0],), device="cuda")
+    m.samples_per_ray[0] = max(m.samples_per_ray[0], 1.3 * int(valid.sum()) / sub.shape[0])
+    m.render_into(sub, rgb, dep)
+    c = m.last_counts()
+    assert c["n_valid"] == int(valid.sum()) and c["overflow"] == 0
+    # rays without a valid sample are background: exactly white, depth 0
+    empty = ~valid.any(-1)
+    assert bool((rgb.cpu()[empty] == 1.0).all()) and bool((dep.cpu()[empty] == 0.0).all())
+
+
+def test_full_frame_oracle_spot_check(gpu_lib, frame):
+    """rgb / depth of the frame's centre block and of a strided sample of the whole frame against the oracle, with
+    the masks of the same rays (the oracle's full render needs the 17 GB of tables on the host)."""
+    p, rays, m = frame
+    centre, _, sparse = _frame_sample(rays)
+    idx = torch.unique(torch.cat([centre, sparse]))
+    sub = rays[idx.cuda()].contiguous()
+    out, _ = m(sub)
+    n_valid = m.last_counts()["n_valid"]
+    ref = O.render_chunk(p.to("cpu"), sub.cpu(), return_aux=True)
+    cull = m.sample_cull(sub)
+    assert torch.equal(cull["ray_valid"].cpu(), ref["ray_valid"]) and n_valid == int(ref["ray_valid"].sum())
+    assert torch.equal(cull["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
+    assert torch.equal(cull["z_vals"].cpu(), ref["z_vals"])
     band = ((ref["weight"] - 1e-3).abs() < 2e-7).any(-1)
-    assert ref["app_mask"].any()
+    assert ref["app_mask"].any() and int(band.sum()) <= 2
     d_rgb = (out["rgb_map"].cpu() - ref["rgb_map"]).abs().max(-1).values
     d_dep = (out["depth_map"].cpu() - ref["depth_map"]).abs()
     assert d_rgb[~band].max().item() <= 1e-4 and d_dep[~band].max().item() <= 1e-4

@@ -506,14 +506,53 @@ def test_appearance_embedding_and_density_projection(gpu_lib):
         _model(_scene(S=64))(rays, app_code=1)
 
 
-def test_render_c1_tiny_config(gpu_lib):
-    """The tiny full-render configuration at reduced image size (the oracle finishes in seconds): the stated
-    init (background only) and the dense variant that runs every stage."""
-    rays = scenes.c1_rays(64, 64)
-    for dense in (False, True):
-        p = scenes.c1_scene(dense=dense)
-        ref, _ = _check_render(p, rays, RGB_TOL_F32)
-        assert bool(ref["app_mask"].any()) == dense
+def _oracle_in_chunks(p, rays, S=-1, chunk=16384):
+    """render_chunk over slices of the rays: rgb, depth, masks and depths of every ray, the rays that hold a weight
+    within rounding of the appearance threshold, and the number of appearance samples."""
+    keep = {k: [] for k in ("rgb_map", "depth_map", "ray_valid", "z_vals", "band")}
+    n_app = 0
+    for i in range(0, rays.shape[0], chunk):
+        r = O.render_chunk(p, rays[i:i + chunk], N_samples=S, return_aux=True)
+        r["band"] = ((r["weight"] - p.rayMarch_weight_thres).abs() < 2e-7).any(-1)
+        n_app += int(r["app_mask"].sum())
+        for k in keep:
+            keep[k].append(r[k])
+    out = {k: torch.cat(v) for k, v in keep.items()}
+    out["n_app"] = n_app
+    return out
+
+
+@pytest.mark.parametrize("dense", [False, True])
+@pytest.mark.parametrize("opt,step_ratio", [(1, 2.0), (0, 0.5), (0, 3.47)])
+def test_render_c1_tiny_config(gpu_lib, opt, step_ratio, dense):
+    """The tiny full-render configuration at its full 400 x 400 image, 128 samples per ray, both samplers: the hull
+    sampler (sampling_opt 1, n_importance 128) and the equal-step sampler (sampling_opt 0, N_samples 128) with the
+    reference's default step_ratio 0.5 (128 steps reach half a scene unit behind the entry point) and with 3.47
+    (the steps span the box diagonal).  Each with the stated init (shift -10: every weight is below the appearance
+    threshold, the image is background) and the dense variant (shift 0) that runs every stage.  Masks, indices and
+    depths bit-exact, rgb / depth within 1e-4."""
+    rays = scenes.c1_rays(400, 400)
+    p = scenes.c1_scene(dense=dense, sampling_opt=opt, step_ratio=step_ratio)
+    assert p.alpha_volume is None and rays.shape[0] == 160000
+    ref = _oracle_in_chunks(p, rays, S=128)
+    assert (ref["n_app"] > 0) == dense and 0 < int(ref["ray_valid"].sum()) < ref["ray_valid"].numel()
+    m = _model(p)
+    cull = m.sample_cull(rays, N_samples=128)
+    assert torch.equal(cull["ray_valid"].cpu(), ref["ray_valid"])
+    assert torch.equal(cull["valid_idx"].cpu(), ref["ray_valid"].reshape(-1).nonzero()[:, 0])
+    assert torch.equal(cull["z_vals"].cpu(), ref["z_vals"])
+    out, _ = m(rays, N_samples=128)
+    assert m.last_counts()["n_valid"] == int(ref["ray_valid"].sum())
+    # rays holding a sample whose weight is within 2e-7 of the appearance threshold may differ by that sample
+    ok = ~ref["band"]
+    assert int(ref["band"].sum()) <= max(3, ref["ray_valid"].numel() // 10000)
+    d_rgb = (out["rgb_map"].cpu() - ref["rgb_map"]).abs().max(-1).values
+    assert d_rgb[ok].max().item() <= RGB_TOL_F32
+    assert (out["depth_map"].cpu() - ref["depth_map"]).abs()[ok].max().item() <= RGB_TOL_F32
+    if ref["band"].any():
+        assert d_rgb[ref["band"]].max().item() <= 2e-3
+    if not dense:
+        assert bool((out["rgb_map"] >= 1.0 - 1e-3).all())
 
 
 def test_render_16bit_network_and_fp16_tables(gpu_lib):

@@ -54,6 +54,33 @@ def test_subfunctions_match_reference(name):
         assert torch.equal(O.sample_alpha(p.alpha_volume, p.alpha_aabb, pts.reshape(-1, 3)), d["sub_alpha_lookup"])
 
 
+@pytest.mark.parametrize("name", NAMES)
+def test_sample_mask_matches_reference_subresults(name):
+    """sample_and_cull's mask = the reference's inside-box mask AND its occupancy lookups above the threshold
+    (both stored in the fixture for every sample), and its depths are the reference sampler's."""
+    p, d, cfg = load_golden(name)
+    xyz, z, valid = O.sample_and_cull(p, d["rays"], cfg["N_samples"])
+    want = d["sub_inside"].bool()
+    if p.alpha_volume is not None:
+        want = want & (d["sub_alpha_lookup"].view(want.shape) > p.alpha_mask_filter_thre)
+    assert torch.equal(valid, want) and torch.equal(z, d["sub_z"]) and torch.equal(xyz, d["sub_pts"])
+    aux = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"], app_code=cfg.get("app_code"), return_aux=True)
+    assert torch.equal(aux["ray_valid"], valid)
+
+
+def test_fixture_masks_are_discriminating():
+    """In several fixtures the occupancy volume removes samples that are inside the box, and keeps others."""
+    culling = 0
+    for name in NAMES:
+        p, d, cfg = load_golden(name)
+        if p.alpha_volume is None:
+            continue
+        inside = d["sub_inside"].bool()
+        keep = d["sub_alpha_lookup"].view(inside.shape) > p.alpha_mask_filter_thre
+        culling += int(bool((inside & ~keep).any()) and bool((inside & keep).any()))
+    assert culling >= 3
+
+
 def test_chunk_driver_is_chunk_invariant():
     p, d, cfg = load_golden("hull_softplus_L1")
     full = O.render_chunk(p, d["rays"], N_samples=cfg["N_samples"])
