@@ -152,3 +152,61 @@ def test_reference_written_files_render_on_the_gpu(gpu_lib, name):
     assert (out["depth_map"].cpu() - d["depth_map"]).abs().max().item() <= 1e-4
     out, _ = m(d["rays"], app_code=cfg["app_code"], N_samples=cfg["N_samples"], white_bg=False)
     assert (out["rgb_map"].cpu() - d["rgb_map_black"]).abs().max().item() <= 1e-4
+
+
+@pytest.mark.gpu
+def test_model_save_writes_the_mask_it_holds(gpu_lib, tmp_path):
+    """GridNeRFHIP.save after updateAlphaMask: the file carries the rebuilt occupancy volume (packed bits, 5-D shape,
+    its box) in the reference's layout (gridnerf_sequential.py:209-223), loads with the weights-only loader, and a
+    model built from it renders what the saving model renders, bit for bit."""
+    from landmark_amd import scenes
+    from landmark_amd.model import GridNeRFHIP
+
+    p = scenes.make_params(seed=21, gridSize=(9, 11, 13), near_far=[0.5, 4.5], n_importance=64, sampling_opt=1,
+                           density_shift=-6.0, step_ratio=0.5, resMode=(1, 2))
+    for t in p.density_plane:
+        t.mul_(8.0)
+    m = GridNeRFHIP(p)
+    assert m.alphaMask is None
+    m.updateAlphaMask(gridSize=(14, 12, 10))
+    vol = m.alphaMask.alpha_volume
+    assert 0 < int(vol.sum()) < vol.numel()
+    path = str(tmp_path / "saved.th")
+    m.save(path)
+    raw = torch.load(path, map_location="cpu", weights_only=False)
+    assert tuple(raw["alphaMask.shape"]) == (1, 1, 10, 12, 14) and raw["alphaMask.mask"].dtype == np.uint8
+    assert set(raw) == {"kwargs", "state_dict", "alphaMask.shape", "alphaMask.mask", "alphaMask.aabb"}
+    q = CK.load_checkpoint(path, sampling_opt=1, n_importance=64)
+    assert torch.equal(q.alpha_volume, vol.reshape(10, 12, 14).cpu()) and torch.equal(q.alpha_aabb, m.alphaMask.aabb.cpu())
+    rays = scenes.pinhole_rays(40, 40, 40.0, scenes.sphere_pose(2.5, 5))
+    a, _ = m(rays)
+    b, _ = GridNeRFHIP(q)(rays)
+    assert torch.equal(a["rgb_map"], b["rgb_map"]) and torch.equal(a["depth_map"], b["depth_map"])
+    released = GridNeRFHIP(scenes.make_params(seed=21, gridSize=(9, 11, 13)), release_source=True)
+    with pytest.raises(Exception, match="released"):
+        released.save(path)
+
+
+@pytest.mark.gpu
+def test_fp16_matrix_modes_refuse_tables_beyond_their_range(gpu_lib):
+    """f16 / f16x2 carry plane x line products as fp16: tables whose products can pass 65504 are refused for those
+    modes at construction (and when the mode is switched), not rendered to inf; bf16 and f32 take them."""
+    from landmark_amd import _lib as L
+    from landmark_amd import scenes
+    from landmark_amd.model import GridNeRFHIP
+
+    p = scenes.make_params(seed=22, gridSize=(9, 11, 13), near_far=[0.5, 4.5], n_importance=64, density_shift=0.0)
+    ok = GridNeRFHIP(p, mlp_precision="f16x2")
+    assert 0 < ok.fp16_range_bounds()["product"] < 1.0
+    p.app_plane[1] = p.app_plane[1] * 3000.0
+    p.app_line[1] = p.app_line[1] * 3000.0
+    for prec in ("f16", "f16x2"):
+        with pytest.raises(L.LandmarkError, match="fp16 range"):
+            GridNeRFHIP(p, mlp_precision=prec)
+    wide = GridNeRFHIP(p, mlp_precision="bf16")
+    rays = scenes.pinhole_rays(24, 24, 24.0, scenes.sphere_pose(2.5, 5))
+    assert bool(torch.isfinite(wide(rays)[0]["rgb_map"]).all())
+    wide.mlp_precision = "f16"
+    with pytest.raises(L.LandmarkError, match="fp16 range"):
+        wide(rays)
+    assert GridNeRFHIP(p, mlp_precision="f16", check_fp16_range=False) is not None

