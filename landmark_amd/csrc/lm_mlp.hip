@@ -31,6 +31,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <utility>
 
 #include "lm_common.h"
 #include "lm_mma.h"
@@ -54,6 +55,22 @@
 #endif
 #ifndef LM_MLP16_NB1
 #define LM_MLP16_NB1 4  // 16-bit modes with one column block: row blocks per pass
+#endif
+
+#ifndef LM_MLP_STREAM
+#define LM_MLP_STREAM 1  // 16-bit and split modes: the layers as one stream of matrix steps (colour_layers_stream)
+#endif
+#ifndef LM_MLP_STREAM_X2
+#define LM_MLP_STREAM_X2 0
+#endif
+#ifndef LM_MLP_PF_X2
+#define LM_MLP_PF_X2 1
+#endif
+#ifndef LM_MLP_PRIO
+#define LM_MLP_PRIO 1  // wave priority while it multiplies (its MFMAs go before the other wave's encoding)
+#endif
+#ifndef LM_MLP_PF
+#define LM_MLP_PF 2  // steps a weight fragment is requested ahead of its MFMAs
 #endif
 
 namespace {
@@ -282,8 +299,10 @@ __device__ __forceinline__ void encode_inputs(const float (*raw)[16],
         float slots[kSlots1];
         constexpr bool kExact = PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2;
         bool big = false;
+        // row 27 / 31 (v = 15) is zero and meets zero weights
+        slots[15] = 0.0f; slots[31] = 0.0f; slots[47] = 0.0f; slots[63] = 0.0f; slots[79] = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
+        for (int v = 0; v < 15; ++v) {
             const float x = raw[cb][v];
             float s1, c1;
             if (PREC == LM_MLP_F16X2) {
@@ -302,7 +321,7 @@ __device__ __forceinline__ void encode_inputs(const float (*raw)[16],
         if (kExact && __builtin_expect(big, 0)) {
             // arguments beyond the fast reduction's range: library routines, rarely if ever taken
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
+            for (int v = 0; v < 15; ++v) {
                 const float x = raw[cb][v];
                 if (fabsf(x) > kSincosMax) {
                     const float s1 = sinf(x), c1 = cosf(x);
@@ -373,6 +392,110 @@ __device__ __forceinline__ void colour_layers(const typename Mma<PREC>::frag *w1
         }
 }
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <typename F, int... I> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// relu of two accumulator values (registers 2 q, 2 q + 1) -> register q % 4 of the next layer's B fragment q / 4
+// (per part)
+template <int PREC>
+__device__ __forceinline__ void relu_pair(const floatx16 &acc, int q, uint32_t (*out)[4]) {
+    using M = Mma<PREC>;
+    uint32_t d[M::NP];
+    if constexpr (PREC == LM_MLP_F16) {
+        // round first, then clamp two halves with one instruction (rounding is monotone and keeps zero)
+        M::pack_pair(acc[2 * q], acc[2 * q + 1], d);
+        const half2v zero = {0, 0};
+        d[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(half2v, d[0]), zero));
+    } else {
+        M::pack_pair(relu_f32(acc[2 * q]), relu_f32(acc[2 * q + 1]), d);
+    }
+#pragma unroll
+    for (int pt = 0; pt < M::NP; ++pt) out[pt][q % 4] = d[pt];
+}
+
+// The three layers of the 16-bit and split modes as one stream of matrix steps.  A "job" is one block of 32 output
+// rows of one layer (4 + 4 + 1 jobs); its NCB accumulators alternate between two register sets, so that the
+// conversion of job j's results (relu, round, split) is issued in small groups behind the MFMAs of job j + 1's first
+// steps and runs under them: a matrix instruction occupies its pipe for 32 cycles while the wave goes on issuing a
+// few ordinary vector instructions.  Once a set's results are converted, the bias of the job after next is read from
+// LDS straight into it, half a job before its first MFMA.  The K order of a layer is the order its inputs become
+// ready in: the last job of a layer is converted while the next layer's first job multiplies the K slices of the
+// earlier jobs.  Weight fragments sit in LDS in exactly this step order (row block, step, part), one pointer walks
+// them; they are requested PF steps ahead, across job and layer boundaries.
+template <int PREC, int NCB, int PF>
+__device__ __forceinline__ void colour_layers_stream(const typename Mma<PREC>::frag *w1, const typename Mma<PREC>::frag *w2,
+                                                     const typename Mma<PREC>::frag *w3, const float *b1, const float *b2,
+                                                     const float *b3,
+                                                     const typename Mma<PREC>::frag (*bfrag)[kSlots1 / Mma<PREC>::G][Mma<PREC>::NP],
+                                                     unsigned lane, float (*out)[3]) {
+    using M = Mma<PREC>;
+    using frag = typename M::frag;
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    constexpr int G = M::G, NP = M::NP;
+    static_assert(G == 8, "eight K slots per lane and step");
+    constexpr int T1 = kSlots1 / G, T2 = 64 / G;
+    constexpr int G1 = 4 * T1, G2 = 4 * T2, GT = G1 + G2 + T2;  // steps of layer 1, layer 2, all
+    constexpr int R = PF + 1;                                    // fragment ring
+    constexpr int PIECES = 2 * NCB;                              // conversion pieces per job: one B fragment each
+    constexpr int NM = NCB * (NP == 2 ? 3 : 1);                  // MFMAs per step
+    const unsigned h = lane >> 5;
+    uint32_t hid1[NCB][T2][NP][4], hid2[NCB][T2][NP][4];
+    floatx16 acc[2][NCB];
+    frag a[R][NP];
+    auto request = [&](int g) {  // g is a constant at every call
+        const frag *p = g < G1 ? w1 + (size_t)g * NP * 64 : (g < G1 + G2 ? w2 + (size_t)(g - G1) * NP * 64 : w3 + (size_t)(g - G1 - G2) * NP * 64);
+#pragma unroll
+        for (int pt = 0; pt < NP; ++pt) a[g % R][pt] = p[pt * 64 + lane];
+    };
+    auto request_bias = [&](int job) {  // into the accumulators of `job`
+        const floatx16 b = load_bias(job < 4 ? b1 : (job < 8 ? b2 : b3), job == 8 ? (int)h : (job & 3) * 2 + (int)h);
+#pragma unroll
+        for (int cb = 0; cb < NCB; ++cb) acc[job & 1][cb] = b;
+    };
+    request_bias(0);
+    static_for<PF>([&](auto gc) { request(decltype(gc)::value); });
+    static_for<GT>([&](auto gc) {
+        constexpr int g = decltype(gc)::value;
+        constexpr int layer = g < G1 ? 0 : (g < G1 + G2 ? 1 : 2);
+        constexpr int job = layer == 0 ? g / T1 : (layer == 1 ? 4 + (g - G1) / T2 : 8);
+        constexpr int t = layer == 0 ? g % T1 : (g - G1) % T2;
+        constexpr int set = job & 1;
+        constexpr bool converting = job > 0 && t >= 1 && t <= PIECES;
+        if constexpr (g + PF < GT) request(g + PF);
+        if constexpr (job < 8 && t == (job == 0 ? 1 : PIECES + 1)) request_bias(job + 1);
+        static_for<NM>([&](auto mc) {
+            constexpr int m = decltype(mc)::value, cb = NP == 2 ? m / 3 : m, part = NP == 2 ? m % 3 : 0;
+            const frag b = layer == 0 ? bfrag[cb][t][part == 2 ? 1 : 0]
+                                      : __builtin_bit_cast(frag, *reinterpret_cast<const u4 *>(layer == 1 ? hid1[cb][t][part == 2 ? 1 : 0] : hid2[cb][t][part == 2 ? 1 : 0]));
+            acc[set][cb] = M::mma(a[g % R][part == 1 ? 1 : 0], b, acc[set][cb]);
+            // the previous job's results: one B fragment per step from the second step on (its last MFMAs have
+            // left the pipe by then), a share of its four registers behind every MFMA of the step
+            if constexpr (converting) {
+                __builtin_amdgcn_sched_barrier(0);  // the MFMA first, the conversions in its shadow
+                constexpr int p = t - 1, pcb = p / 2, u = p % 2, prev = job - 1;
+                constexpr int q0 = 4 * m / NM, q1 = 4 * (m + 1) / NM;
+                auto *dst = prev < 4 ? hid1[pcb][2 * prev + u] : hid2[pcb][2 * (prev - 4) + u];
+#pragma unroll
+                for (int q = q0; q < q1; ++q) relu_pair<PREC>(acc[set ^ 1][pcb], 4 * u + q, dst);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        });
+        __builtin_amdgcn_sched_barrier(0);
+    });
+#pragma unroll
+    for (int cb = 0; cb < NCB; ++cb)
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const float e = PREC == LM_MLP_F16X2 ? expf(-acc[0][cb][k]) : __expf(-acc[0][cb][k]);
+            out[cb][k] = __builtin_amdgcn_rcpf(1.0f + e);
+        }
+}
+
 template <int PREC> struct LdsPlan {
     using M = Mma<PREC>;
     static constexpr size_t kW1 = (size_t)4 * kSlots1 * 64 * sizeof(typename M::elem) * M::NP;
@@ -381,7 +504,15 @@ template <int PREC> struct LdsPlan {
     static constexpr bool kW3InLds = (kW1 + kW2 + kW3) <= 96 * 1024;
     static constexpr size_t kBias = (4 * 2 * 16 + 4 * 2 * 16 + 2 * 16) * sizeof(float);  // b1 | b2 | b3, register order
     static constexpr size_t kWeights = kW1 + kW2 + (kW3InLds ? kW3 : 0);
-    static constexpr size_t kBytes = kWeights + kBias;
+    static constexpr size_t kQueue = kWeights + kBias;  // the workgroup's tile counter
+    // 16-bit modes: every wave owns a staging area that receives its next tile's feature rows (27 floats per row,
+    // contiguous in memory) straight from global memory, rounded up to whole 1 KB transfers
+    static constexpr bool kStaged = LM_MLP_STREAM && (PREC == LM_MLP_F16 || PREC == LM_MLP_BF16);
+    static constexpr size_t kTileBytes = (size_t)32 * MlpBlock<PREC>::NCB * kAppDim * sizeof(float);
+    static constexpr size_t kStageWave = (kTileBytes + 1023) / 1024 * 1024;
+    static constexpr size_t kStage = kQueue + 16;
+    static constexpr size_t kBytes = kStage + (kStaged ? kStageWave * (MlpBlock<PREC>::N / LM_WAVE) : 0);
+    static_assert(kBytes <= 160 * 1024, "LDS of a compute unit");
 };
 
 template <int PREC>
@@ -402,6 +533,7 @@ __device__ __forceinline__ void stage_weights(char *lds, const char *packed, con
     const float *b1 = (const float *)(packed + L.b1), *b2 = (const float *)(packed + L.b2), *b3 = (const float *)(packed + L.b3);
     for (unsigned i = threadIdx.x; i < 128; i += blockDim.x) { bl[i] = b1[i]; bl[128 + i] = b2[i]; }
     for (unsigned i = threadIdx.x; i < 32; i += blockDim.x) bl[256 + i] = b3[i];
+    if (threadIdx.x == 0) *reinterpret_cast<uint32_t *>(lds + P::kQueue) = blockDim.x / LM_WAVE;  // one tile per wave is dealt at the start
     __syncthreads();
 }
 
@@ -429,7 +561,6 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
     constexpr int NCB = MlpBlock<PREC>::NCB, TILE = 32 * NCB;
     const uint64_t n_tiles = (M + TILE - 1) / TILE;
     const unsigned wpb = MlpBlock<PREC>::N / LM_WAVE;
-    const uint64_t wave_id = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * wpb + threadIdx.x / LM_WAVE;
     const uint64_t n_waves = (uint64_t)gridDim.x * wpb;
     // The lane's 16 input rows (features, view direction, zeros) of its sample in each column block.  Half h
     // holds rows row_of(v, 0) + 4 h: features up to row 23, then rows 24..26 (features, h = 0) or 28..30 (the
@@ -469,23 +600,126 @@ __global__ __launch_bounds__(MlpBlock<PREC>::N) void k_mlp(const char *__restric
             raw[cb][15] = 0.0f;
         }
     };
-    // A tile's inputs are encoded into the first layer's fragments first; the registers that held them then
-    // receive the next tile's inputs, which travel while this tile is multiplied.
     constexpr int T1 = kSlots1 / Mm::G;
     float raw[NCB][16];
-    if (wave_id < n_tiles) fetch(wave_id, raw);
-    for (uint64_t tile = wave_id; tile < n_tiles; tile += n_waves) {
-        frag bfrag[NCB][T1][Mm::NP];
-        encode_inputs<PREC, NCB>(raw, bfrag);
-        if (tile + n_waves < n_tiles) fetch(tile + n_waves, raw);
-        float out[NCB][3];
-        colour_layers<PREC, NCB>(w1, w2, w3, b1, b2, b3, bfrag, lane, out);
+    // Tiles are dealt to workgroups in rounds of one tile per wave; inside a workgroup a wave takes the group's next
+    // tile from a counter in LDS when it has encoded its current one.  The SIMD issues its oldest wave first, so its
+    // two waves advance at different speeds, and with a fixed share per wave the slower one would finish alone.
+    uint32_t *queue = reinterpret_cast<uint32_t *>(lds + P::kQueue);
+    const uint64_t first = (uint64_t)lm_xcd_swizzle(blockIdx.x, gridDim.x) * wpb;
+    auto tile_of = [&](uint32_t q) { return (uint64_t)(q / wpb) * n_waves + first + q % wpb; };
+    auto claim = [&]() {
+        uint32_t q = 0;
+        if (lane == 0) q = atomicAdd(queue, 1u);
+        return tile_of(__builtin_amdgcn_readfirstlane(q));
+    };
+    uint64_t tile = tile_of(threadIdx.x / LM_WAVE);
+    if constexpr (P::kStaged) {
+        // The feature rows of a tile are one contiguous run of global memory: the wave copies it into its staging
+        // area with transfers that bypass the registers (16 bytes per lane, 1 KB per instruction; 4-byte transfers
+        // when the array is not 16-byte aligned) while the previous tile is multiplied, and every lane picks its
+        // 12 or 15 values from LDS when the tile's turn comes.  Only the view direction (three values of the
+        // lanes of the upper half) travels through registers.
+        char *stage = lds + P::kStage + (threadIdx.x / LM_WAVE) * P::kStageWave;
+        const float *stage_f = reinterpret_cast<const float *>(stage);
+        const bool wide = (reinterpret_cast<uintptr_t>(feat) & 15u) == 0;
+        typedef const void __attribute__((address_space(1))) *gptr;
+        typedef void __attribute__((address_space(3))) *lptr;
+        float vdir[NCB][3];
+        auto request = [&](uint64_t t) {
+            // Lanes whose share lies beyond the tile or the array repeat the last valid transfer (into their own
+            // part of the staging area, which nobody reads): no lane is switched off, no branch.
+            const uint64_t begin = t * P::kTileBytes, left = M * (kAppDim * sizeof(float)) - begin;
+            const unsigned span = (unsigned)(left < P::kTileBytes ? left : P::kTileBytes);
+            const char *src = reinterpret_cast<const char *>(feat) + begin;
+            if (wide) {
+                const unsigned last = ((span + 15u) & ~15u) - 16u;
 #pragma unroll
-        for (int cb = 0; cb < NCB; ++cb) {
-            const uint64_t p = tile * TILE + cb * 32 + j;
-            if (p < M && h == 0) {
-                rgb[p * 3 + 0] = out[cb][0]; rgb[p * 3 + 1] = out[cb][1]; rgb[p * 3 + 2] = out[cb][2];
+                for (unsigned k = 0; k < P::kStageWave / 1024; ++k) {
+                    const unsigned off = (k * 64 + lane) * 16;
+                    __builtin_amdgcn_global_load_lds((gptr)(src + (off < last ? off : last)), (lptr)(stage + k * 1024), 16, 0, 0);
+                }
+            } else {
+                const unsigned last = span - 4u;
+#pragma unroll 1
+                for (unsigned k = 0; k < P::kTileBytes / 256; ++k) {
+                    const unsigned off = (k * 64 + lane) * 4;
+                    __builtin_amdgcn_global_load_lds((gptr)(src + (off < last ? off : last)), (lptr)(stage + k * 256), 4, 0, 0);
+                }
             }
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const uint64_t p = t * TILE + cb * 32 + j;
+                const uint64_t pc = p < M ? p : M - 1;
+                const float *vsrc = MODE == 0 ? view + pc * 3 : view + 6 * (size_t)(app_idx[pc] / (uint32_t)S) + 3;
+#pragma unroll
+                for (int k = 0; k < 3; ++k) vdir[cb][k] = vsrc[k];
+            }
+        };
+        if (tile < n_tiles) request(tile);
+        float out[NCB][3];
+        uint64_t done = ~0ull;  // the tile whose colours wait in `out`
+        auto store = [&]() {
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const uint64_t p = done * TILE + cb * 32 + j;
+                if (done != ~0ull && p < M && h == 0) {
+                    rgb[p * 3 + 0] = out[cb][0]; rgb[p * 3 + 1] = out[cb][1]; rgb[p * 3 + 2] = out[cb][2];
+                }
+            }
+        };
+        while (tile < n_tiles) {
+            const uint64_t next = claim();
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the transfers into the staging area have landed
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const float *r = stage_f + (cb * 32 + j) * kAppDim;
+#pragma unroll
+                for (int v = 0; v < 12; ++v) raw[cb][v] = r[4 * h + row_of(v, 0)];
+#pragma unroll
+                for (int v = 12; v < 15; ++v) raw[cb][v] = h ? vdir[cb][v - 12] : r[12 + v];
+                raw[cb][15] = 0.0f;
+            }
+            // the previous tile's colours leave now, so that the wait above never waits for them
+            store();
+            frag bfrag[NCB][T1][Mm::NP];
+            encode_inputs<PREC, NCB>(raw, bfrag);
+            // every lane holds its values in registers: the staging area may be overwritten
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if (next < n_tiles) request(next);
+            __builtin_amdgcn_sched_barrier(0);
+#if LM_MLP_PRIO
+            __builtin_amdgcn_s_setprio(LM_MLP_PRIO);
+#endif
+            colour_layers_stream<PREC, NCB, LM_MLP_PF>(w1, w2, w3, b1, b2, b3, bfrag, lane, out);
+#if LM_MLP_PRIO
+            __builtin_amdgcn_s_setprio(0);
+#endif
+            done = tile;
+            tile = next;
+        }
+        store();
+    } else {
+        // A tile's inputs are encoded into the first layer's fragments first; the registers that held them then
+        // receive the next tile's inputs, which travel while this tile is multiplied.
+        if (tile < n_tiles) fetch(tile, raw);
+        while (tile < n_tiles) {
+            frag bfrag[NCB][T1][Mm::NP];
+            encode_inputs<PREC, NCB>(raw, bfrag);
+            const uint64_t next = claim();
+            if (next < n_tiles) fetch(next, raw);
+            float out[NCB][3];
+            if constexpr (PREC == LM_MLP_F16X2 && LM_MLP_STREAM_X2) colour_layers_stream<PREC, NCB, LM_MLP_PF_X2>(w1, w2, w3, b1, b2, b3, bfrag, lane, out);
+            else colour_layers<PREC, NCB>(w1, w2, w3, b1, b2, b3, bfrag, lane, out);
+#pragma unroll
+            for (int cb = 0; cb < NCB; ++cb) {
+                const uint64_t p = tile * TILE + cb * 32 + j;
+                if (p < M && h == 0) {
+                    rgb[p * 3 + 0] = out[cb][0]; rgb[p * 3 + 1] = out[cb][1]; rgb[p * 3 + 2] = out[cb][2];
+                }
+            }
+            tile = next;
         }
     }
 }

@@ -51,6 +51,13 @@ template <> struct Mma<LM_MLP_F16> {
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[0][i] = (_Float16)s[i];
     }
+    // two values -> one register of the operand (per part)
+    __device__ static __forceinline__ void pack_pair(float x0, float x1, uint32_t *o) {
+        half2v h;
+        h[0] = (_Float16)x0;
+        h[1] = (_Float16)x1;
+        o[0] = __builtin_bit_cast(uint32_t, h);
+    }
 };
 template <> struct Mma<LM_MLP_BF16> {
     static constexpr int G = 8, CW = 8, NP = 1;
@@ -62,6 +69,13 @@ template <> struct Mma<LM_MLP_BF16> {
     __device__ static __forceinline__ void pack(const float *s, frag *o) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[0][i] = (__bf16)s[i];
+    }
+    __device__ static __forceinline__ void pack_pair(float x0, float x1, uint32_t *o) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        bf16x2 h;
+        h[0] = (__bf16)x0;
+        h[1] = (__bf16)x1;
+        o[0] = __builtin_bit_cast(uint32_t, h);
     }
 };
 template <> struct Mma<LM_MLP_F16X2> {
@@ -76,20 +90,26 @@ template <> struct Mma<LM_MLP_F16X2> {
     // an operand, the result rounded to fp16 into the low or the high half) gives lo: three instructions per
     // pair instead of the seven the compiler makes of the scalar expression (convert, convert back, subtract,
     // convert, per value, plus packing).
+    __device__ static __forceinline__ void pack_pair(float x0, float x1, uint32_t *o) {
+        half2v h;
+        h[0] = (_Float16)x0;
+        h[1] = (_Float16)x1;
+        const uint32_t hb = __builtin_bit_cast(uint32_t, h);
+        uint32_t l;
+        asm("v_fma_mixlo_f16 %0, %1, -1.0, %2 op_sel_hi:[1,0,0]" : "=v"(l) : "v"(hb), "v"(x0));
+        asm("v_fma_mixhi_f16 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(l) : "v"(hb), "v"(x1));
+        o[0] = hb;
+        o[1] = l;
+    }
     __device__ static __forceinline__ void pack(const float *s, frag *o) {
         typedef uint32_t u4 __attribute__((ext_vector_type(4)));
         u4 hi, lo;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            half2v h;
-            h[0] = (_Float16)s[2 * i];
-            h[1] = (_Float16)s[2 * i + 1];
-            const uint32_t hb = __builtin_bit_cast(uint32_t, h);
-            uint32_t l;
-            asm("v_fma_mixlo_f16 %0, %1, -1.0, %2 op_sel_hi:[1,0,0]" : "=v"(l) : "v"(hb), "v"(s[2 * i]));
-            asm("v_fma_mixhi_f16 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(l) : "v"(hb), "v"(s[2 * i + 1]));
-            hi[i] = hb;
-            lo[i] = l;
+            uint32_t d[2];
+            pack_pair(s[2 * i], s[2 * i + 1], d);
+            hi[i] = d[0];
+            lo[i] = d[1];
         }
         o[0] = __builtin_bit_cast(half8, hi);
         o[1] = __builtin_bit_cast(half8, lo);
