@@ -14,6 +14,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 SO_PATH = os.path.join(HERE, "liblandmark_hip.so")
+MICROBENCH_PATH = os.path.join(HERE, "build", "mfma_valu_coissue")
 SOURCES = ["lm_api.hip", "lm_sample.hip", "lm_gather.hip", "lm_mlp.hip", "lm_composite.hip", "lm_frame.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
@@ -47,6 +48,9 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
         raise RuntimeError("hipcc failed")
     link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", SO_PATH, *objs]
     subprocess.check_call(link)
+    # the micro-benchmark the colour network's schedule rests on (a program of its own, not part of the library)
+    subprocess.check_call([hipcc, "--offload-arch=gfx950", "-O3", "-w", os.path.join(CSRC, "microbench", "mfma_valu_coissue.hip"),
+                           "-o", MICROBENCH_PATH])
     if verbose:
         print(f"[build] wrote {SO_PATH}")
     return SO_PATH

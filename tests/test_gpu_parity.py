@@ -273,6 +273,26 @@ def test_colour_network(gpu_lib, prec, tol):
         assert (got - ref).abs().max().item() < tol, (M, prec)
 
 
+@pytest.mark.parametrize("prec,tol", [("f16", 4e-3), ("bf16", 3e-2)])
+@pytest.mark.parametrize("shift", [0, 1, 2, 3])
+def test_colour_network_staged_inputs(gpu_lib, prec, tol, shift):
+    """The 16-bit modes copy a tile's feature rows into LDS with 16-byte transfers, or 4-byte ones when the feature
+    array does not start on a 16-byte boundary (here: a view that starts `shift` floats into its storage), and a
+    workgroup's waves take tiles from a shared counter: row counts around whole tiles, around one round of tiles over
+    all workgroups and above it, every row checked."""
+    p = scenes.make_params(seed=5, gridSize=(4, 4, 4), density_n_comp=4, app_n_comp=48)
+    m = _model(p)
+    g = torch.Generator().manual_seed(16 + shift)
+    for M in (63, 64, 65, 127, 8 * 256 * 64 - 1, 8 * 256 * 64 + 129):
+        store = torch.randn(M * 27 + shift, generator=g).to("cuda")
+        feats = store[shift:].view(M, 27)
+        assert feats.data_ptr() % 16 == (4 * shift) % 16
+        view = torch.randn(M, 3, generator=g)
+        got = m.render_module(view, feats, precision=prec).cpu()
+        ref = O.mlp_render(p, view, feats.cpu())
+        assert (got - ref).abs().max().item() < tol, (M, prec, shift)
+
+
 @pytest.mark.parametrize("prec", ["f32", "f16x2"])
 def test_colour_network_large_arguments(gpu_lib, prec):
     """Features far outside the fast sine / cosine reduction's range (|x| > 8192) take the library routines: the
