@@ -43,7 +43,7 @@
 #define LM_MLP_NCB 2
 #endif
 // split-fp16 mode: eight waves with one column block each beat four waves with two (the second wave of a SIMD
-// covers the first one's waits for LDS and memory; vector and matrix instructions themselves do not overlap)
+// covers the first one's waits for LDS and memory)
 #ifndef LM_MLPX2_THREADS
 #define LM_MLPX2_THREADS 512
 #endif
@@ -479,7 +479,9 @@ __device__ __forceinline__ void colour_layers_stream(const typename Mma<PREC>::f
                 __builtin_amdgcn_sched_barrier(0);  // the MFMA first, the conversions in its shadow
                 constexpr int p = t - 1, pcb = p / 2, u = p % 2, prev = job - 1;
                 constexpr int q0 = 4 * m / NM, q1 = 4 * (m + 1) / NM;
-                auto *dst = prev < 4 ? hid1[pcb][2 * prev + u] : hid2[pcb][2 * (prev - 4) + u];
+                uint32_t(*dst)[4];
+                if constexpr (prev < 4) dst = hid1[pcb][2 * prev + u];
+                else dst = hid2[pcb][2 * (prev - 4) + u];
 #pragma unroll
                 for (int q = q0; q < q1; ++q) relu_pair<PREC>(acc[set ^ 1][pcb], 4 * u + q, dst);
                 __builtin_amdgcn_sched_barrier(0);
