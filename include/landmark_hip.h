@@ -37,7 +37,7 @@ extern "C" {
 
 /* Changes whenever a struct, an enum value or the meaning of an argument does (2: 16-word counter block;
  * 3: workspace capacities in lm_model, LM_STAT_OVERFLOW). */
-#define LM_ABI_VERSION 3
+#define LM_ABI_VERSION 4
 #define LM_MAX_PLANES 12 /* ndims * len(resMode) */
 
 typedef enum lm_status {
@@ -110,6 +110,10 @@ typedef struct lm_geom {
      * up to float rounding; here the lookup reads block b alone (difference below 1e-6 relative). */
     int32_t div0, div1;
     float blk_w, blk_h;
+    /* Optional coarse level of a cell table (vol_dtype LM_CELLS), built by lm_pack_occupancy_coarse; NULL = none.
+     * It lets the culling kernels reject runs of samples that lie in empty space without visiting them; the
+     * decisions are the same with and without it. */
+    const uint8_t *vol_coarse;
 } lm_geom;
 
 /* stages of lm_render, in launch order */
@@ -191,6 +195,14 @@ int lm_relayout_nchw_to_hwc(const void *src, void *dst, int32_t C, int32_t H, in
  * structure for AlphaGridMask.sample_alpha (app/models/alpha_mask.py:35-47). */
 int lm_pack_occupancy(const float *vol, int32_t D, int32_t H, int32_t W, uint8_t *cells, uint32_t *not_binary,
                       void *stream);
+
+/* Coarse level of a cell table: one byte per block of 8 x 8 x 8 cells, set when any cell of the block or of its
+ * upper neighbours (+1 block along every axis) has a bit set, so that one lookup answers for a run of samples that
+ * spans at most two blocks per axis.  coarse: lm_occupancy_coarse_bytes(D, H, W) bytes.  No counterpart in the
+ * reference: an acceleration structure for AlphaGridMask.sample_alpha (app/models/alpha_mask.py:35-47) at the
+ * reference's default of half a grid cell per sample (gridnerf_sequential.py:244-281). */
+size_t lm_occupancy_coarse_bytes(int32_t D, int32_t H, int32_t W);
+int lm_pack_occupancy_coarse(const uint8_t *cells, int32_t D, int32_t H, int32_t W, uint8_t *coarse, void *stream);
 
 /* Alpha of a segment of length `length` at the gx*gy*gz lattice points
  * aabb0*(1-s) + aabb1*s, s taken from the device tables lin_x[gx], lin_y[gy], lin_z[gz]

@@ -15,7 +15,7 @@ LM_MAX_PLANES = 12
 LM_STATIC_WORKSPACE_BYTES = 80 << 20
 LM_N_STAGES = 6
 STAGE_NAMES = ["cull", "density_march", "app_list", "app_gather", "colour", "composite"]
-LM_ABI_VERSION = 3  # include/landmark_hip.h
+LM_ABI_VERSION = 4  # include/landmark_hip.h
 LM_STAT_N_VALID, LM_STAT_N_APP, LM_STAT_N_MARCHED, LM_STAT_OVERFLOW, LM_STAT_BINS, LM_STAT_QUEUE, LM_STAT_WORDS = 0, 1, 2, 3, 4, 8, 16
 LM_F32, LM_F16, LM_U8, LM_CELLS = 0, 1, 2, 3
 LM_SAMPLER_AABB, LM_SAMPLER_HULL = 0, 1
@@ -39,6 +39,7 @@ class LmGeom(C.Structure):
         ("vol", C.c_void_p), ("vd", C.c_int32), ("vh", C.c_int32), ("vw", C.c_int32), ("vol_dtype", C.c_int32),
         ("vol_aabb_min", C.c_float * 3), ("vol_inv", C.c_float * 3), ("vol_thre", C.c_float),
         ("div0", C.c_int32), ("div1", C.c_int32), ("blk_w", C.c_float), ("blk_h", C.c_float),
+        ("vol_coarse", C.c_void_p),
     ]
 
 
@@ -60,6 +61,8 @@ SYMBOLS = {
     "lm_last_error": (C.c_char_p, []),
     "lm_relayout_nchw_to_hwc": (C.c_int, [_P, _P, _I32, _I32, _I32, _I32, _P]),
     "lm_pack_occupancy": (C.c_int, [_P, _I32, _I32, _I32, _P, _P, _P]),
+    "lm_occupancy_coarse_bytes": (_SZ, [_I32, _I32, _I32]),
+    "lm_pack_occupancy_coarse": (C.c_int, [_P, _I32, _I32, _I32, _P, _P]),
     "lm_dense_alpha": (C.c_int, [C.POINTER(LmModel), _P, _P, _P, _I32, _I32, _I32, _F, _P, _P]),
     "lm_alpha_mask_pool": (C.c_int, [_P, _I32, _I32, _I32, _F, _P, _P, _P, _P]),
     "lm_sample_cull_scratch_bytes": (_SZ, [_I64, _I32]),

@@ -79,39 +79,120 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *
 // same few cache lines (a wave of 64 samples along one ray touches 64 different ones), and the
 // per-ray work (slab test or hull distance) is done once per word instead of once per sample.
 // A workgroup covers 256 consecutive words = 4 of the 64-word groups k_scan_blocks counts.
+// Bounds of the points of samples s0 .. s0 + n - 1 of one ray: they lie between the first and the last one (the depth
+// tables are monotone, and so is o + d * z in z), widened by a margin a hundred times the rounding of the operations
+// involved.  lo[k] <= pt[k] <= hi[k] for every sample of the run; NaNs propagate into the bounds.
+__device__ __forceinline__ void run_bounds(const lm_geom &g, const float *ray, float rp, int s0, int n, float *lo, float *hi) {
+    const float za = lm_sample_z(g, rp, s0), zb = lm_sample_z(g, rp, s0 + n - 1);
+    const float zlo = fminf(za, zb), zhi = fmaxf(za, zb);
+    // the depth is a sum of two terms bounded by |near| and the ray's parameter (or by the depth itself)
+    const float zm = 1e-5f * (fmaxf(fabsf(zlo), fabsf(zhi)) + fabsf(rp) + fabsf(g.near_));
+    const bool z_nan = !(za == za) || !(zb == zb);  // fminf / fmaxf would drop a NaN
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        const float o = ray[k], d = ray[3 + k];
+        const float e0 = d * (zlo - zm), e1 = d * (zhi + zm), e2 = d * (zlo + zm), e3 = d * (zhi - zm);
+        const float l = o + fminf(fminf(e0, e1), fminf(e2, e3)), h = o + fmaxf(fmaxf(e0, e1), fmaxf(e2, e3));
+        const float m = 1e-5f * (fabsf(o) + fmaxf(fabsf(l), fabsf(h))) + 1e-30f;
+        const bool bad = z_nan || !(e0 == e0) || !(e1 == e1) || !(e2 == e2) || !(e3 == e3);
+        lo[k] = bad ? NAN : l - m;
+        hi[k] = bad ? NAN : h + m;
+    }
+}
+
+// 1: every point within the bounds fails the box test (it stays on the outer side of one face).  Anything doubtful
+// (NaN included) is 0.
+__device__ __forceinline__ bool bounds_outside(const lm_geom &g, const float *lo, const float *hi) {
+    bool outside = false;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) outside |= (hi[k] < g.aabb[k]) | (lo[k] > g.aabb[3 + k]);
+    return outside;
+}
+
+// The coarse level of a cell table (lm_pack_occupancy_coarse): blocks of 8 x 8 x 8 cells, entry b set when a cell of
+// blocks b .. b + 1 (per axis) has a bit set.
+constexpr int kCoarseShift = 3;
+__host__ __device__ inline int coarse_dim(int cells) { return (cells + (1 << kCoarseShift) - 1) >> kCoarseShift; }
+
+// Cell index range of the points within the bounds, per axis, with lm_cells_positive's own float operations: each of
+// them is monotone (weakly, rounding included) in the coordinate when vol_inv > 0, so the floor of a point's cell
+// coordinate lies between the floors of the bounds'.  Returns 0 when the bounds hold a NaN or the volume is degenerate
+// (no statement), 1 with the block range [b0, b1] per axis otherwise; `none` = every index is outside the table
+// (all samples are rejected by the lookup itself).
+__device__ __forceinline__ bool coarse_range(const lm_geom &g, const float *lo, const float *hi, int *b0, int *b1, bool &none) {
+    const int dims[3] = {g.vw, g.vh, g.vd};
+    none = false;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        if (!(lo[k] <= hi[k]) || !(g.vol_inv[k] > 0.0f) || dims[k] < 2) return false;
+        const float s = (float)(dims[k] - 1);
+        float il = (((lo[k] - g.vol_aabb_min[k]) * g.vol_inv[k] - 1.0f) + 1.0f) / 2.0f * s;
+        float ih = (((hi[k] - g.vol_aabb_min[k]) * g.vol_inv[k] - 1.0f) + 1.0f) / 2.0f * s;
+        if (!(il <= ih)) return false;
+        il = fminf(fmaxf(floorf(il), -2.0f), (float)dims[k]);
+        ih = fminf(fmaxf(floorf(ih), -2.0f), (float)dims[k]);
+        // cell index = floor + 1; indices outside 0 .. dims fail the lookup's range test
+        int c0 = (int)il + 1, c1 = (int)ih + 1;
+        if (c1 < 0 || c0 > dims[k]) none = true;
+        c0 = max(c0, 0);
+        c1 = min(c1, dims[k]);
+        b0[k] = c0 >> kCoarseShift;
+        b1[k] = c1 >> kCoarseShift;
+    }
+    return true;
+}
+
+// 1: no sample of the run can pass the cell lookup (every cell it can fall into is empty, or lies outside the table)
+__device__ __forceinline__ bool coarse_empty(const lm_geom &g, const float *lo, const float *hi, int &span) {
+    int b0[3], b1[3];
+    bool none;
+    span = INT_MAX;
+    if (!coarse_range(g, lo, hi, b0, b1, none)) return false;
+    if (none) return true;
+    span = max(max(b1[0] - b0[0], b1[1] - b0[1]), b1[2] - b0[2]);
+    if (span > 1) return false;
+    const int nx = coarse_dim(g.vw + 1), ny = coarse_dim(g.vh + 1);
+    return g.vol_coarse[((size_t)b0[2] * ny + b0[1]) * nx + b0[0]] == 0;
+}
+
 // Decisions of samples s0 .. s0 + n - 1 (n <= 64) of one ray, sample s0 + i in bit bit0 + i.
 __device__ __forceinline__ uint64_t segment_bits(const lm_geom &g, const float *ray, float rp, int s0, int n, int bit0) {
-    // The samples lie between the first and the last one (the depth tables are monotone, and so is
-    // o + d * z in z).  If that segment, widened by a margin a hundred times the rounding of the
-    // operations involved, stays on the outer side of one face of the box, every sample fails the box
-    // test and the bits are zero without visiting them.  Anything doubtful (NaN included) is visited.
-    {
-        const float za = lm_sample_z(g, rp, s0), zb = lm_sample_z(g, rp, s0 + n - 1);
-        const float zlo = fminf(za, zb), zhi = fmaxf(za, zb);
-        // the depth is a sum of two terms bounded by |near| and the ray's parameter (or by the depth itself)
-        const float zm = 1e-5f * (fmaxf(fabsf(zlo), fabsf(zhi)) + fabsf(rp) + fabsf(g.near_));
-        bool outside = false;
-#pragma unroll
-        for (int k = 0; k < 3; ++k) {
-            const float o = ray[k], d = ray[3 + k];
-            const float e0 = d * (zlo - zm), e1 = d * (zhi + zm), e2 = d * (zlo + zm), e3 = d * (zhi - zm);
-            const float lo = o + fminf(fminf(e0, e1), fminf(e2, e3)), hi = o + fmaxf(fmaxf(e0, e1), fmaxf(e2, e3));
-            const float m = 1e-5f * (fabsf(o) + fmaxf(fabsf(lo), fabsf(hi))) + 1e-30f;
-            outside |= (hi + m < g.aabb[k]) | (lo - m > g.aabb[3 + k]);
-        }
-        if (outside) return 0ull;
-    }
+    // A run whose bounds stay outside the box has no valid sample, and neither has one whose cells are all empty:
+    // the bits are zero without visiting the samples.
     const bool cells0 = g.vol && g.vol_dtype == LM_CELLS && g.vol_thre == 0.0f;
+    const bool coarse = cells0 && g.vol_coarse;
+    bool pieces = false;
+    {
+        float lo[3], hi[3];
+        run_bounds(g, ray, rp, s0, n, lo, hi);
+        if (bounds_outside(g, lo, hi)) return 0ull;
+        if (coarse) {
+            int span;
+            if (coarse_empty(g, lo, hi, span)) return 0ull;
+            // quarters of the run have a chance when the whole run spans few blocks
+            pieces = n >= 32 && span <= 6;
+        }
+    }
     uint64_t bits = 0;
+    const int step = pieces ? (n + 3) / 4 : n;
+    for (int p0 = 0; p0 < n; p0 += step) {
+        const int pn = min(step, n - p0);
+        if (pieces) {
+            float lo[3], hi[3];
+            int span;
+            run_bounds(g, ray, rp, s0 + p0, pn, lo, hi);
+            if (bounds_outside(g, lo, hi) || coarse_empty(g, lo, hi, span)) continue;
+        }
 #pragma unroll 4
-    for (int i = 0; i < n; ++i) {
-        const float z = lm_sample_z(g, rp, s0 + i);
-        float pt[3];
-        lm_point(ray, z, pt);
-        bool ok;
-        if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
-        else ok = lm_sample_valid(g, pt);
-        bits |= (uint64_t)ok << (bit0 + i);
+        for (int i = p0; i < p0 + pn; ++i) {
+            const float z = lm_sample_z(g, rp, s0 + i);
+            float pt[3];
+            lm_point(ray, z, pt);
+            bool ok;
+            if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
+            else ok = lm_sample_valid(g, pt);
+            bits |= (uint64_t)ok << (bit0 + i);
+        }
     }
     return bits;
 }
@@ -342,6 +423,30 @@ __global__ __launch_bounds__(kBlock) void k_emit(const uint64_t *__restrict__ bi
     }
 }
 
+// coarse level, step 1: any[b] = some cell of block b has a bit set
+__global__ __launch_bounds__(256) void k_coarse_any(const uint8_t *__restrict__ cells, int D1, int H1, int W1, uint8_t *__restrict__ any) {
+    const int nx = coarse_dim(W1), ny = coarse_dim(H1), nz = coarse_dim(D1);
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)nx * ny * nz) return;
+    const int bx = (int)(i % nx), by = (int)((i / nx) % ny), bz = (int)(i / ((size_t)nx * ny));
+    unsigned acc = 0;
+    for (int z = bz << kCoarseShift; z < min((bz + 1) << kCoarseShift, D1); ++z)
+        for (int y = by << kCoarseShift; y < min((by + 1) << kCoarseShift, H1); ++y)
+            for (int x = bx << kCoarseShift; x < min((bx + 1) << kCoarseShift, W1); ++x) acc |= cells[((size_t)z * H1 + y) * W1 + x];
+    any[i] = acc ? 1 : 0;
+}
+// step 2: coarse[b] = any over blocks b .. b + 1 along every axis
+__global__ __launch_bounds__(256) void k_coarse_dilate(const uint8_t *__restrict__ any, int nz, int ny, int nx, uint8_t *__restrict__ coarse) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)nx * ny * nz) return;
+    const int bx = (int)(i % nx), by = (int)((i / nx) % ny), bz = (int)(i / ((size_t)nx * ny));
+    unsigned acc = 0;
+    for (int z = bz; z < min(bz + 2, nz); ++z)
+        for (int y = by; y < min(by + 2, ny); ++y)
+            for (int x = bx; x < min(bx + 2, nx); ++x) acc |= any[((size_t)z * ny + y) * nx + x];
+    coarse[i] = acc ? 1 : 0;
+}
+
 __global__ __launch_bounds__(256) void k_pack_occupancy(const float *__restrict__ vol, int D, int H, int W,
                                                         uint8_t *__restrict__ cells, uint32_t *__restrict__ not_binary) {
     const size_t n = (size_t)(D + 1) * (H + 1) * (W + 1);
@@ -503,6 +608,24 @@ extern "C" int lm_pack_occupancy(const float *vol, int32_t D, int32_t H, int32_t
     hipLaunchKernelGGL(k_pack_occupancy, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, vol, D, H, W,
                        cells, not_binary);
     LM_CHECK_LAUNCH("k_pack_occupancy");
+    return LM_OK;
+}
+
+// The coarse table and, behind it, the undilated one it is made from (scratch of the build): 2 n bytes.
+extern "C" size_t lm_occupancy_coarse_bytes(int32_t D, int32_t H, int32_t W) {
+    if (D <= 0 || H <= 0 || W <= 0) return 0;
+    return 2 * (size_t)coarse_dim(D + 1) * coarse_dim(H + 1) * coarse_dim(W + 1);
+}
+
+extern "C" int lm_pack_occupancy_coarse(const uint8_t *cells, int32_t D, int32_t H, int32_t W, uint8_t *coarse, void *stream) {
+    LM_REQUIRE(cells && coarse, "null buffer");
+    LM_REQUIRE(D > 0 && H > 0 && W > 0, "empty volume");
+    const int nz = coarse_dim(D + 1), ny = coarse_dim(H + 1), nx = coarse_dim(W + 1);
+    const size_t n = (size_t)nx * ny * nz;
+    uint8_t *any = coarse + n;
+    hipLaunchKernelGGL(k_coarse_any, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, cells, D + 1, H + 1, W + 1, any);
+    hipLaunchKernelGGL(k_coarse_dilate, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, any, nz, ny, nx, coarse);
+    LM_CHECK_LAUNCH("k_coarse_dilate");
     return LM_OK;
 }
 

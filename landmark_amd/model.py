@@ -46,6 +46,7 @@ class GridNeRFHIP:
         term_eps: float = 0.0,
         release_source: bool = False,
         occupancy: str = "auto",  # auto | cells | u8 | f32: storage of the occupancy volume
+        coarse_occupancy: bool = True,  # a coarse level over the cell table: empty runs of samples are skipped
         capacity: str = "adaptive",  # adaptive | worst: how the render workspace is sized (see `capacities`)
         check_fp16_range: bool = True,  # refuse f16 / f16x2 for tables whose products can leave the fp16 range
     ):
@@ -83,6 +84,7 @@ class GridNeRFHIP:
         self.gridSize = list(params.gridSize)
         self.stepSize = params.stepSize
         self._occupancy = occupancy
+        self._coarse_occupancy = bool(coarse_occupancy)
         self._geom_cache: Dict[int, Tuple[L.LmGeom, tuple]] = {}
         self._struct_cache: Dict[tuple, L.LmModel] = {}
         self._need_cache: Dict[tuple, int] = {}
@@ -153,6 +155,7 @@ class GridNeRFHIP:
         self._invalidate()
         self.alphaMask = None
         self._vol, self._vol_store, self._vol_dtype, self._alpha_aabb = None, None, L.LM_F32, None
+        self._vol_coarse = None
         if volume is None:
             return
         vol = volume.to(self.device, torch.float32).contiguous()
@@ -167,6 +170,10 @@ class GridNeRFHIP:
             if self._occupancy != "u8" and int(flag.item()) == 0:
                 # a 0/1 mask (what the reference stores): one byte per trilinear cell, one load per sample
                 self._vol_dtype, self._vol_store = L.LM_CELLS, cells
+                if self._coarse_occupancy:
+                    coarse = torch.empty(self.lib.lm_occupancy_coarse_bytes(D, H, W), dtype=torch.uint8, device=self.device)
+                    L.check(self.lib.lm_pack_occupancy_coarse(cells.data_ptr(), D, H, W, coarse.data_ptr(), L.current_stream()), "lm_pack_occupancy_coarse")
+                    self._vol_coarse = coarse
             else:
                 as_u8 = self._vol.clamp(0, 255).to(torch.uint8)
                 if bool((as_u8.float() == self._vol).all()):
@@ -322,6 +329,8 @@ class GridNeRFHIP:
         if self._vol is not None:
             g.vol = self._vol_store.data_ptr()
             g.vol_dtype = self._vol_dtype
+            if self._vol_coarse is not None:
+                g.vol_coarse = self._vol_coarse.data_ptr()
             g.vd, g.vh, g.vw = self._vol.shape[-3:]
             ab = self._alpha_aabb
             g.vol_aabb_min[:] = ab[0].tolist()

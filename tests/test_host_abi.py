@@ -39,7 +39,7 @@ def test_every_declared_symbol_is_exported(lib):
 
 def test_struct_sizes_match_header_layout():
     assert C.sizeof(L.LmPlane) == 48
-    assert C.sizeof(L.LmGeom) == 144  # 40 B scalars, 2 pointers, inv_aabb + pad, pointer, 4 ints, 7 floats + pad
+    assert C.sizeof(L.LmGeom) == 152  # 40 B scalars, 2 pointers, inv_aabb + pad, pointer, 4 ints, 7 floats, 2 ints, 2 floats, pointer
     assert C.sizeof(L.LmModel) % 8 == 0
 
 
