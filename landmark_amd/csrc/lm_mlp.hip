@@ -447,10 +447,23 @@ __device__ __forceinline__ void colour_layers_stream(const typename Mma<PREC>::f
     uint32_t hid1[NCB][T2][NP][4], hid2[NCB][T2][NP][4];
     floatx16 acc[2][NCB];
     frag a[R][NP];
-    auto request = [&](int g) {  // g is a constant at every call
-        const frag *p = g < G1 ? w1 + (size_t)g * NP * 64 : (g < G1 + G2 ? w2 + (size_t)(g - G1) * NP * 64 : w3 + (size_t)(g - G1 - G2) * NP * 64);
+    // The fragments of the layers lie one behind the other in LDS (w2 follows w1, w3 follows w2 where it is resident),
+    // in the order of the steps: a running offset walks them, advanced once per request and hidden from the compiler,
+    // which would otherwise form one address register per fragment beyond the 64 KB an instruction's offset reaches,
+    // lift them all out of the tile loop and spill them.
+    const bool w3_follows = w3 == w2 + (size_t)G2 * NP * 64;
+    uint32_t walk = lane, walk3 = lane;  // in fragments
+    auto request = [&](int g) {  // g is a constant at every call; requests come in the order of g
+        const frag *p = (g < G1 + G2 || w3_follows) ? w1 + walk : w3 + walk3;
 #pragma unroll
-        for (int pt = 0; pt < NP; ++pt) a[g % R][pt] = p[pt * 64 + lane];
+        for (int pt = 0; pt < NP; ++pt) a[g % R][pt] = p[pt * 64];
+        if (g < G1 + G2 || w3_follows) {
+            walk += NP * 64;
+            asm volatile("" : "+v"(walk));
+        } else {
+            walk3 += NP * 64;
+            asm volatile("" : "+v"(walk3));
+        }
     };
     auto request_bias = [&](int job) {  // into the accumulators of `job`
         const floatx16 b = load_bias(job < 4 ? b1 : (job < 8 ? b2 : b3), job == 8 ? (int)h : (job & 3) * 2 + (int)h);
