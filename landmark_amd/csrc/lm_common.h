@@ -1,5 +1,6 @@
 // Shared declarations of the gfx950 kernels behind include/landmark_hip.h.
 #pragma once
+#include <utility>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -231,6 +232,14 @@ __device__ __forceinline__ bool lm_sample_valid(const lm_geom &g, const float *p
     bool ok = lm_inside(g, pt);
     if (ok && g.vol) ok = lm_alpha_lookup(g, pt) > g.vol_thre;
     return ok;
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <typename F, int... I> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // ---------------------------------------------------------------------------------------

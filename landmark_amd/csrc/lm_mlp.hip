@@ -31,7 +31,6 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
-#include <utility>
 
 #include "lm_common.h"
 #include "lm_mma.h"
@@ -390,14 +389,6 @@ __device__ __forceinline__ void colour_layers(const typename Mma<PREC>::frag *w1
             const float e = (PREC == LM_MLP_F32 || PREC == LM_MLP_F16X2) ? expf(-acc3[0][cb][k]) : __expf(-acc3[0][cb][k]);
             out[cb][k] = __builtin_amdgcn_rcpf(1.0f + e);
         }
-}
-
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
-template <typename F, int... I> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
-    static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 // relu of two accumulator values (registers 2 q, 2 q + 1) -> register q % 4 of the next layer's B fragment q / 4
