@@ -432,7 +432,6 @@ __device__ __forceinline__ void colour_layers_stream(const typename Mma<PREC>::f
     constexpr int T1 = kSlots1 / G, T2 = 64 / G;
     constexpr int G1 = 4 * T1, G2 = 4 * T2, GT = G1 + G2 + T2;  // steps of layer 1, layer 2, all
     constexpr int R = PF + 1;                                    // fragment ring
-    constexpr int PIECES = 2 * NCB;                              // conversion pieces per job: one B fragment each
     constexpr int NM = NCB * (NP == 2 ? 3 : 1);                  // MFMAs per step
     const unsigned h = lane >> 5;
     uint32_t hid1[NCB][T2][NP][4], hid2[NCB][T2][NP][4];
@@ -469,25 +468,33 @@ __device__ __forceinline__ void colour_layers_stream(const typename Mma<PREC>::f
         constexpr int job = layer == 0 ? g / T1 : (layer == 1 ? 4 + (g - G1) / T2 : 8);
         constexpr int t = layer == 0 ? g % T1 : (g - G1) % T2;
         constexpr int set = job & 1;
-        constexpr bool converting = job > 0 && t >= 1 && t <= PIECES;
+        // conversion slots: PPM register pairs behind every MFMA from the second step on, until the previous job's
+        // 8 NCB pairs are done
+        constexpr int PPM = NP == 2 ? 1 : 2, PAIRS = 8 * NCB;
+        constexpr int TC = (PAIRS + PPM * NM - 1) / (PPM * NM);  // steps the conversions take
+        constexpr bool converting = job > 0 && t >= 1 && t <= TC;
         if constexpr (g + PF < GT) request(g + PF);
-        if constexpr (job < 8 && t == (job == 0 ? 1 : PIECES + 1)) request_bias(job + 1);
+        if constexpr (job < 8 && t == (job == 0 ? 1 : TC + 1)) request_bias(job + 1);
         static_for<NM>([&](auto mc) {
             constexpr int m = decltype(mc)::value, cb = NP == 2 ? m / 3 : m, part = NP == 2 ? m % 3 : 0;
             const frag b = layer == 0 ? bfrag[cb][t][part == 2 ? 1 : 0]
                                       : __builtin_bit_cast(frag, *reinterpret_cast<const u4 *>(layer == 1 ? hid1[cb][t][part == 2 ? 1 : 0] : hid2[cb][t][part == 2 ? 1 : 0]));
             acc[set][cb] = M::mma(a[g % R][part == 1 ? 1 : 0], b, acc[set][cb]);
-            // the previous job's results: one B fragment per step from the second step on (its last MFMAs have
-            // left the pipe by then), a share of its four registers behind every MFMA of the step
+            // the previous job's results, from the second step on (its last MFMAs have left the pipe by then): a few
+            // register pairs behind every MFMA; pair w of the job belongs to B fragment w / 4 = (column block, half)
             if constexpr (converting) {
                 __builtin_amdgcn_sched_barrier(0);  // the MFMA first, the conversions in its shadow
-                constexpr int p = t - 1, pcb = p / 2, u = p % 2, prev = job - 1;
-                constexpr int q0 = 4 * m / NM, q1 = 4 * (m + 1) / NM;
-                uint32_t(*dst)[4];
-                if constexpr (prev < 4) dst = hid1[pcb][2 * prev + u];
-                else dst = hid2[pcb][2 * (prev - 4) + u];
-#pragma unroll
-                for (int q = q0; q < q1; ++q) relu_pair<PREC>(acc[set ^ 1][pcb], 4 * u + q, dst);
+                constexpr int slot = (t - 1) * NM + m, prev = job - 1;
+                static_for<PPM>([&](auto wc) {
+                    constexpr int w = slot * PPM + decltype(wc)::value;
+                    if constexpr (w < PAIRS) {
+                        constexpr int piece = w / 4, pcb = piece / 2, u = piece % 2;
+                        uint32_t(*dst)[4];
+                        if constexpr (prev < 4) dst = hid1[pcb][2 * prev + u];
+                        else dst = hid2[pcb][2 * (prev - 4) + u];
+                        relu_pair<PREC>(acc[set ^ 1][pcb], 4 * u + w % 4, dst);
+                    }
+                });
                 __builtin_amdgcn_sched_barrier(0);
             }
         });
