@@ -81,20 +81,23 @@ __global__ __launch_bounds__(kBlock) void k_sample_cull(lm_geom g, const float *
 // A workgroup covers 256 consecutive words = 4 of the 64-word groups k_scan_blocks counts.
 // Bounds of the points of samples s0 .. s0 + n - 1 of one ray: they lie between the first and the last one (the depth
 // tables are monotone, and so is o + d * z in z), widened by a margin a hundred times the rounding of the operations
-// involved.  lo[k] <= pt[k] <= hi[k] for every sample of the run; NaNs propagate into the bounds.
+// involved.  lo[k] <= pt[k] <= hi[k] for every sample of the run.  fminf / fmaxf drop NaNs; with FLAG_NAN a NaN anywhere
+// on the way makes the bounds NaN (for the cell test, which must make no statement then; the box test needs no flag:
+// what its bounds miss fails the per-sample test as well).
+template <bool FLAG_NAN>
 __device__ __forceinline__ void run_bounds(const lm_geom &g, const float *ray, float rp, int s0, int n, float *lo, float *hi) {
     const float za = lm_sample_z(g, rp, s0), zb = lm_sample_z(g, rp, s0 + n - 1);
     const float zlo = fminf(za, zb), zhi = fmaxf(za, zb);
     // the depth is a sum of two terms bounded by |near| and the ray's parameter (or by the depth itself)
     const float zm = 1e-5f * (fmaxf(fabsf(zlo), fabsf(zhi)) + fabsf(rp) + fabsf(g.near_));
-    const bool z_nan = !(za == za) || !(zb == zb);  // fminf / fmaxf would drop a NaN
+    const bool z_nan = FLAG_NAN && (!(za == za) || !(zb == zb));
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
         const float o = ray[k], d = ray[3 + k];
         const float e0 = d * (zlo - zm), e1 = d * (zhi + zm), e2 = d * (zlo + zm), e3 = d * (zhi - zm);
         const float l = o + fminf(fminf(e0, e1), fminf(e2, e3)), h = o + fmaxf(fmaxf(e0, e1), fmaxf(e2, e3));
         const float m = 1e-5f * (fabsf(o) + fmaxf(fabsf(l), fabsf(h))) + 1e-30f;
-        const bool bad = z_nan || !(e0 == e0) || !(e1 == e1) || !(e2 == e2) || !(e3 == e3);
+        const bool bad = FLAG_NAN && (z_nan || !(e0 == e0) || !(e1 == e1) || !(e2 == e2) || !(e3 == e3));
         lo[k] = bad ? NAN : l - m;
         hi[k] = bad ? NAN : h + m;
     }
@@ -164,7 +167,8 @@ __device__ __forceinline__ uint64_t segment_bits(const lm_geom &g, const float *
     bool pieces = false;
     {
         float lo[3], hi[3];
-        run_bounds(g, ray, rp, s0, n, lo, hi);
+        if (coarse) run_bounds<true>(g, ray, rp, s0, n, lo, hi);
+        else run_bounds<false>(g, ray, rp, s0, n, lo, hi);
         if (bounds_outside(g, lo, hi)) return 0ull;
         if (coarse) {
             int span;
@@ -174,17 +178,9 @@ __device__ __forceinline__ uint64_t segment_bits(const lm_geom &g, const float *
         }
     }
     uint64_t bits = 0;
-    const int step = pieces ? (n + 3) / 4 : n;
-    for (int p0 = 0; p0 < n; p0 += step) {
-        const int pn = min(step, n - p0);
-        if (pieces) {
-            float lo[3], hi[3];
-            int span;
-            run_bounds(g, ray, rp, s0 + p0, pn, lo, hi);
-            if (bounds_outside(g, lo, hi) || coarse_empty(g, lo, hi, span)) continue;
-        }
+    auto visit = [&](int i0, int i1) {
 #pragma unroll 4
-        for (int i = p0; i < p0 + pn; ++i) {
+        for (int i = i0; i < i1; ++i) {
             const float z = lm_sample_z(g, rp, s0 + i);
             float pt[3];
             lm_point(ray, z, pt);
@@ -192,6 +188,19 @@ __device__ __forceinline__ uint64_t segment_bits(const lm_geom &g, const float *
             if (cells0) ok = lm_inside(g, pt) && lm_cells_positive(g, pt);
             else ok = lm_sample_valid(g, pt);
             bits |= (uint64_t)ok << (bit0 + i);
+        }
+    };
+    if (!pieces) {
+        visit(0, n);  // n is a constant for most callers: the loop unrolls without a remainder
+    } else {
+        const int step = (n + 3) / 4;
+        for (int p0 = 0; p0 < n; p0 += step) {
+            const int pn = min(step, n - p0);
+            float lo[3], hi[3];
+            int span;
+            run_bounds<true>(g, ray, rp, s0 + p0, pn, lo, hi);
+            if (bounds_outside(g, lo, hi) || coarse_empty(g, lo, hi, span)) continue;
+            visit(p0, p0 + pn);
         }
     }
     return bits;

@@ -329,7 +329,7 @@ class GridNeRFHIP:
         if self._vol is not None:
             g.vol = self._vol_store.data_ptr()
             g.vol_dtype = self._vol_dtype
-            if self._vol_coarse is not None:
+            if self._vol_coarse is not None and self._coarse_can_act(S):
                 g.vol_coarse = self._vol_coarse.data_ptr()
             g.vd, g.vh, g.vw = self._vol.shape[-3:]
             ab = self._alpha_aabb
@@ -343,6 +343,19 @@ class GridNeRFHIP:
             g.blk_h = torch.tensor(2 / g.div1, dtype=torch.float32).item()
         self._geom_cache[S] = (g, (a_d, t_d))
         return g
+
+    def _coarse_can_act(self, S: int) -> bool:
+        """The coarse occupancy level answers for runs of 16 samples that span at most two blocks of 8 cells per axis:
+        it is handed to the kernels when neighbouring samples are at most about a cell apart (the equal-step sampler's
+        step, or the hull sampler's longest spacing (far - near) / (S - 1)), and left out where it could only cost."""
+        p = self.p
+        ab = self._alpha_aabb
+        cell = float(((ab[1] - ab[0]) / torch.tensor([float(d - 1) for d in self._vol.shape[-3:]][::-1]).clamp(min=1.0)).min())
+        if p.sampling_opt == 0:
+            spacing = float(torch.as_tensor(p.stepSize).item())
+        else:
+            spacing = (float(p.near_far[1]) - float(p.near_far[0])) / max(S - 1, 1)
+        return spacing <= 1.25 * cell
 
     def _model_struct(self, S: int, white_bg: bool, caps: Tuple[int, int] = (0, 0)) -> L.LmModel:
         """The lm_model of a render with S samples per ray and workspace capacities `caps` (valid samples,
