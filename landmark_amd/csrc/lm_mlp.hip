@@ -402,6 +402,13 @@ __device__ __forceinline__ void relu_pair(const floatx16 &acc, int q, uint32_t (
         M::pack_pair(acc[2 * q], acc[2 * q + 1], d);
         const half2v zero = {0, 0};
         d[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(half2v, d[0]), zero));
+    } else if constexpr (PREC == LM_MLP_BF16) {
+        // round first, then clamp both halves with one packed integer maximum: a negative bf16 number is a negative
+        // 16-bit integer, a non-negative one keeps its bits
+        typedef short short2v __attribute__((ext_vector_type(2)));
+        M::pack_pair(acc[2 * q], acc[2 * q + 1], d);
+        const short2v zero = {0, 0};
+        d[0] = __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(short2v, d[0]), zero));
     } else {
         M::pack_pair(relu_f32(acc[2 * q]), relu_f32(acc[2 * q + 1]), d);
     }
@@ -442,15 +449,20 @@ __device__ __forceinline__ void colour_layers_stream(const typename Mma<PREC>::f
     // which would otherwise form one address register per fragment beyond the 64 KB an instruction's offset reaches,
     // lift them all out of the tile loop and spill them.
     const bool w3_follows = w3 == w2 + (size_t)G2 * NP * 64;
-    uint32_t walk = lane, walk3 = lane;  // in fragments
+    typedef const frag __attribute__((address_space(3))) *lds_frag;
+    uint32_t walk = (uint32_t)(uintptr_t)(lds_frag)w1 + lane * (uint32_t)sizeof(frag);  // LDS byte address
+    uint32_t walk3 = lane;                                                            // fragments of w3 in global memory
     auto request = [&](int g) {  // g is a constant at every call; requests come in the order of g
-        const frag *p = (g < G1 + G2 || w3_follows) ? w1 + walk : w3 + walk3;
-#pragma unroll
-        for (int pt = 0; pt < NP; ++pt) a[g % R][pt] = p[pt * 64];
         if (g < G1 + G2 || w3_follows) {
-            walk += NP * 64;
+            const lds_frag p = (lds_frag)(uintptr_t)walk;
+#pragma unroll
+            for (int pt = 0; pt < NP; ++pt) a[g % R][pt] = p[pt * 64];
+            walk += NP * 64 * (uint32_t)sizeof(frag);
             asm volatile("" : "+v"(walk));
         } else {
+            const frag *p = w3 + walk3;
+#pragma unroll
+            for (int pt = 0; pt < NP; ++pt) a[g % R][pt] = p[pt * 64];
             walk3 += NP * 64;
             asm volatile("" : "+v"(walk3));
         }

@@ -66,16 +66,24 @@ template <> struct Mma<LM_MLP_BF16> {
     __device__ static __forceinline__ floatx16 mma(frag a, frag b, floatx16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
-    __device__ static __forceinline__ void pack(const float *s, frag *o) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[0][i] = (__bf16)s[i];
-    }
+    // two values -> one register with one packed conversion (converted one by one, the compiler emits a packed
+    // conversion per value and a byte permute per pair)
     __device__ static __forceinline__ void pack_pair(float x0, float x1, uint32_t *o) {
         typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        bf16x2 h;
-        h[0] = (__bf16)x0;
-        h[1] = (__bf16)x1;
-        o[0] = __builtin_bit_cast(uint32_t, h);
+        typedef float float2v __attribute__((ext_vector_type(2)));
+        const float2v v = {x0, x1};
+        o[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+    }
+    __device__ static __forceinline__ void pack(const float *s, frag *o) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t d;
+            pack_pair(s[2 * i], s[2 * i + 1], &d);
+            r[i] = d;
+        }
+        o[0] = __builtin_bit_cast(bf16x8, r);
     }
 };
 template <> struct Mma<LM_MLP_F16X2> {
