@@ -233,6 +233,24 @@ def test_gather_matches_grid_sample(gpu_lib, ndims, res, dn, an):
     assert torch.allclose(got_a, ref_a, atol=2e-6)
 
 
+@pytest.mark.parametrize("an,dtype,M", [(8, torch.float32, 3), (24, torch.float32, 1001), (72, torch.float32, 257),
+                                        (72, torch.float16, 530), (40, torch.float16, 77), (64, torch.float16, 15),
+                                        (48, torch.float32, 16), (80, torch.float32, 4099)])
+def test_app_products_other_widths_and_counts(gpu_lib, an, dtype, M):
+    """The stage-level appearance gather writes a wave's sixteen samples through an LDS tile (planes of up to 64
+    channels) or directly (wider planes): channel counts on both sides of that limit and off the multiples of 16 (six
+    planes, so that their sum stays a multiple of 16 as basis_mat's packing asks), row
+    counts that leave a wave partly filled or a workgroup with idle waves."""
+    p = scenes.make_params(seed=11, gridSize=(9, 14, 6), ndims=3, resMode=(1, 2), density_n_comp=8, app_n_comp=an,
+                           feature_init="uniform", dtype=dtype)
+    g = torch.Generator().manual_seed(12)
+    xyz = torch.rand(M, 3, generator=g) * 2.1 - 1.05
+    got = _model(p).app_products(xyz).cpu()
+    ref = O.app_products(p, xyz)
+    assert got.shape == ref.shape == (M, 6 * an)
+    assert torch.allclose(got, ref, atol=2e-6)
+
+
 def test_gather_fp16_tables(gpu_lib):
     p = scenes.make_params(seed=9, gridSize=(17, 12, 10), ndims=3, resMode=(1, 2), density_n_comp=16, app_n_comp=48,
                            dtype=torch.float16)
