@@ -440,6 +440,17 @@ def _check_render(p, rays, tol, S=-1, white_bg=True, **kw):
     return ref, out
 
 
+@pytest.mark.parametrize("an,dn,dtype,tol", [(24, 8, torch.float32, RGB_TOL_F32), (40, 12, torch.float32, RGB_TOL_F32),
+                                             (80, 16, torch.float32, RGB_TOL_F32), (24, 8, torch.float16, 1e-2)])
+def test_render_other_channel_counts(gpu_lib, an, dn, dtype, tol):
+    """Appearance planes whose channel count is not 16, 32, 48 or 64 leave the fused gather: the render forms the
+    plane x line product matrix in memory and projects it with basis_mat in a second kernel.  Same picture."""
+    p = _scene(seed=21, S=96, shift=0.0, ndims=3, resMode=(1, 2), app_n_comp=an, density_n_comp=dn, dtype=dtype)
+    rays = scenes.pinhole_rays(48, 40, 42.0, scenes.sphere_pose(2.5, 4))
+    ref, _ = _check_render(p, rays, tol, S=96)
+    assert ref["app_mask"].any()
+
+
 @pytest.mark.parametrize("name", golden_names())
 def test_render_golden_vectors(gpu_lib, name):
     p, d, cfg = load_golden(name)
