@@ -101,6 +101,16 @@ def test_argument_validation_returns_status_not_abort(lib):
     assert rc == -1 and b"2^31" in lib.lm_last_error()
 
 
+def test_coarse_occupancy_sizes_and_validation(lib):
+    """Two tables of one byte per block of 8 x 8 x 8 cells (the coarse level and the undilated one it is built from);
+    null buffers and empty volumes are refused before anything is launched."""
+    assert lib.lm_occupancy_coarse_bytes(256, 256, 256) == 2 * 33 ** 3
+    assert lib.lm_occupancy_coarse_bytes(7, 8, 64) == 2 * 1 * 2 * 9
+    assert lib.lm_occupancy_coarse_bytes(0, 8, 8) == 0
+    assert lib.lm_pack_occupancy_coarse(None, 8, 8, 8, None, None) == -1 and b"null" in lib.lm_last_error()
+    assert lib.lm_pack_occupancy_coarse(16, 0, 8, 8, 16, None) == -1 and b"empty" in lib.lm_last_error()
+
+
 def _host_model(S=128, C=48, n=3):
     """An lm_model good enough for size queries (pointers are never dereferenced on the host)."""
     m = L.LmModel()
