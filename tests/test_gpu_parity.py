@@ -761,6 +761,26 @@ def test_early_termination_bounds(gpu_lib, fp16_tables, res):
     assert (term["depth_map"] - exact["depth_map"]).abs().max().item() <= 1e-4 * 4.5 * 1.5
 
 
+@pytest.mark.parametrize("prec", ["f32", "f16x2"])
+def test_termination_at_the_benchmark_rule_keeps_the_parity_bar(gpu_lib, prec):
+    """bench.py stops a ray at T < 1e-4 / far, chosen so that neither rgb (<= eps with a white background) nor depth
+    (<= eps * far) can move by more than the fp32 bar: rendered with that value the picture still meets the bar against
+    the oracle, which never stops a ray, and the appearance samples are the same ones."""
+    p = _scene(S=128, resMode=(1, 2))
+    rays = scenes.pinhole_rays(48, 48, 40.0, scenes.sphere_pose(2.5, 5))
+    eps = 1e-4 / float(p.near_far[1])
+    m = _model(p, term_eps=eps, mlp_precision=prec)
+    got, _ = m(rays)
+    ref = O.render_chunk(p, rays)
+    assert (got["rgb_map"].cpu() - ref["rgb_map"]).abs().max().item() <= RGB_TOL_F32
+    assert (got["depth_map"].cpu() - ref["depth_map"]).abs().max().item() <= RGB_TOL_F32
+    n_app = m.last_counts()["n_app"]
+    m0 = _model(p, mlp_precision=prec)
+    exact, _ = m0(rays)
+    assert n_app == m0.last_counts()["n_app"] > 0
+    assert (got["rgb_map"] - exact["rgb_map"]).abs().max().item() <= eps + 1e-6
+
+
 def test_ray_generation_and_rgba8(gpu_lib):
     from landmark_amd.render import generate_rays, postprocess_rgba8
 
