@@ -345,6 +345,23 @@ def bench_frame(args, workload):
             c1 = frame_chunks(m1, N, S, W, args.chunk, not args.no_row_hint)
             out["ms_per_step_P1"] = {"workload": f"c4_1080p_multires_P1_base{args.base}_shift{args.density_shift:g}",
                                      "ms": timed_complete(m1, c1, "one-orientation model")}
+            del m1, p1
+            torch.cuda.empty_cache()
+        # the shape most of the reference's run configurations use (one orientation, three levels, equal-step AABB
+        # sampler, appearance embedding, basis_den) on the same tables, mask and camera, at two and at half a grid cell
+        # per step (the reference's default); `--workload prod` times it stage by stage
+        out["ms_per_step_production_shape"] = {}
+        for step_ratio in (2.0, 0.5):
+            pp = scenes.production_scene(base=args.base, step_ratio=step_ratio, device=dev, density_shift=args.density_shift)
+            mp = GridNeRFHIP(pp, device=dev, mlp_precision=args.mlp, term_eps=1e-4 / float(pp.near_far[1]), release_source=True)
+            mp._set_app_code(args.mlp, 3)
+            Sp = mp._samples_for(-1)
+            cp = frame_chunks(mp, N, Sp, W, args.chunk, not args.no_row_hint)
+            steps = 3
+            out["ms_per_step_production_shape"][f"step_ratio_{step_ratio:g}"] = {
+                "samples_per_ray": Sp, "ms": timed_complete(mp, cp, f"production shape, step ratio {step_ratio:g}")}
+            del mp, pp
+            torch.cuda.empty_cache()
     return out
 
 
