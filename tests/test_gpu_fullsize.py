@@ -176,6 +176,38 @@ def test_full_frame_sample_masks_bit_exact(gpu_lib, frame):
     assert bool((rgb.cpu()[empty] == 1.0).all()) and bool((dep.cpu()[empty] == 0.0).all())
 
 
+def test_production_shape_full_size_against_oracle(gpu_lib):
+    """The shape most of the reference's run configurations use (one orientation at three levels, the equal-step
+    AABB sampler at its default of half a grid cell per step = 3544 samples per ray, appearance embedding, density
+    projection) on the benchmark frame's occupancy volume and camera, where the coarse occupancy level acts on every
+    ray: masks, index list and depths of 8 000 rays spread over the frame equal the oracle's bit for bit, the
+    whole-chunk render counts the oracle's valid and appearance samples, and its pixels meet the fp32 bar."""
+    p = scenes.production_scene(base=1024, step_ratio=0.5, device="cuda")
+    rays = scenes.c4_rays(1080, 1920, device="cuda")
+    m = _model(p, mlp_precision="f16x2")
+    assert m._samples_for(-1) == 3544 and m._coarse_can_act(3544)
+    idx = torch.arange(0, 1080 * 1920, 257)
+    sub = rays[idx.cuda()].contiguous()
+    ref = O.render_chunk(p.to("cpu"), sub.cpu(), return_aux=True, app_code=3)
+    valid = ref["ray_valid"]
+    assert 0.001 < valid.float().mean().item() < 0.5
+    cull = m.sample_cull(sub)
+    assert torch.equal(cull["ray_valid"].cpu(), valid)
+    assert torch.equal(cull["valid_idx"].cpu(), valid.reshape(-1).nonzero()[:, 0])
+    assert torch.equal(cull["z_vals"].cpu(), ref["z_vals"])
+    out, _ = m(sub, app_code=3)
+    c = m.last_counts()
+    band = ((ref["weight"] - p.rayMarch_weight_thres).abs() < 2e-7).any(-1)
+    assert c["n_valid"] == int(valid.sum()) and c["overflow"] == 0
+    assert abs(c["n_app"] - int(ref["app_mask"].sum())) <= int(band.sum())
+    ok = ~band
+    assert (out["rgb_map"].cpu() - ref["rgb_map"])[ok].abs().max().item() <= 1e-4
+    assert (out["depth_map"].cpu() - ref["depth_map"])[ok].abs().max().item() <= 1e-4
+    off = _model(p, mlp_precision="f16x2", coarse_occupancy=False)
+    plain, _ = off(sub, app_code=3)
+    assert torch.equal(plain["rgb_map"], out["rgb_map"]) and torch.equal(plain["depth_map"], out["depth_map"])
+
+
 def test_full_frame_oracle_spot_check(gpu_lib, frame):
     """rgb / depth of the frame's centre block and of a strided sample of the whole frame against the oracle, with
     the masks of the same rays (the oracle's full render needs the 17 GB of tables on the host)."""
